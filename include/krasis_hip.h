@@ -383,6 +383,15 @@ typedef struct {
      * norm_bias: the norms carry a bias tensor beside their weight.  All zero with residual_mult 1 and pre_norm 1 = one pre-normed parallel block. */
     int block_kind, pre_norm, post_norm, norm_bias;
     float residual_mult;
+    /* ---- further block mechanisms (all zero = off) */
+    int norm_groups;            /* > 1: every norm splits the row into this many equal consecutive parts and norms each by its own statistics */
+    float embed_scale;          /* 0 or 1: the embedding row as it is; else x = embed[token] * embed_scale */
+    int canon_taps;             /* > 1: the mixer reads h + conv(h) instead of h, a causal convolution over the request's positions on each channel
+                                 * (tensor canon [width, taps]: conv(h)_t = sum_j w[:, j] h_(t - taps + 1 + j), zeros before position 0); the last
+                                 * taps - 1 rows h of every request are part of its state, in every layer */
+    int res_gate;               /* 1: a sublayer's output is multiplied by sigmoid(W h + b) before it joins the stream; h = the sublayer's (normed) input
+                                 * before the input convolution; tensors res_gate1 / res_gate1_b (mixer), res_gate2 / res_gate2_b (feed-forward).
+                                 * Sequential pre-normed blocks only */
 } kr_serve_config;
 typedef struct {
     /* mixer: attention over the paged cache; the feed-forward follows it or runs beside it (kr_serve_config.block_kind) */
@@ -396,7 +405,7 @@ typedef struct {
     int kv_from;                       /* -1, or the earlier layer whose cached keys / values this layer attends to (no k / v projections of its own) */
     int mlp_kind;
     int ff, dense_act;                 /* dense: down(act(gate h, up h)) */
-    int experts, top, groups, keep, renorm;   /* router: softmax over all experts; best `keep` of `groups` groups; `top` experts; weights = scores */
+    int experts, top, groups, keep, renorm;   /* router: scores over all experts; best `keep` of `groups` groups; `top` experts; weights = scores (renorm: / (their sum + 1e-20)) */
     int expert_ff, expert_act; float expert_limit, expert_alpha;
     int shared_ff; float shared_limit;        /* 0 = no shared expert */
     /* ---- mechanisms a design may switch on beside the ones above (all zero = off) */
@@ -410,15 +419,40 @@ typedef struct {
     int chunk;                         /* position i sees j <= i with floor(i / chunk) == floor(j / chunk); 0 = off (not together with window) */
     int dist_bias; float dist_bias_exp;        /* score -= slope_h * (i - j), slope_h = 2^(-dist_bias_exp * (h + 1) / heads) */
     int v_mix;                         /* KR_SERVE_VMIX_*: values blended with the values an earlier layer formed for the same token, before they are cached */
-    int router_bias;                   /* router logits + bias[expert] before the selection */
+    int router_bias;                   /* KR_SERVE_RBIAS_*: bias[expert] joins the logits before everything, or the scores for the choice only */
+    /* ---- attention */
+    int proj_bias;                     /* q, k and the output projection carry biases (tensors q_bias, k_bias, o_bias) */
+    int v_from_k;                      /* the values are the keys as projected (with their bias, before any norm); no v projection; vdim == dim */
+    float softcap;                     /* > 0: score <- softcap * tanh(score / softcap), after the scale, before the distance bias */
+    int out_gate;                      /* KR_SERVE_OGATE_*: the mixer's output is gated by a projection of the mixer's input (tensor out_gate) before W_o */
+    /* ---- recurrent mixers (KR_SERVE_MIX_RETENTION, KR_SERVE_MIX_MLSTM): a matrix state S [dim, vdim] per head and request slot, f32, carried from
+     * token to token; heads x dim queries and keys, heads x vdim values (kv_heads == heads); rotation (rot_*) applies to q and k of a retention layer */
+    float gate_cap;                    /* mlstm: gate pre-activations z <- gate_cap * tanh(z / gate_cap) (0 = uncapped) */
+    int lin_norm_weight;               /* the per-head RMS norm of the mixer's output is followed by a weight [heads * vdim] (tensor lin_norm) */
+    /* ---- router */
+    int router_score;                  /* KR_SERVE_RSCORE_SOFTMAX | KR_SERVE_RSCORE_SIGMOID */
+    int group_score;                   /* KR_SERVE_GSCORE_MAX (a group's largest choice score) | KR_SERVE_GSCORE_TOP2 (the sum of its two largest) */
 } kr_serve_layer;
 #define KR_SERVE_BLOCK_PARALLEL 0
 #define KR_SERVE_BLOCK_SEQUENTIAL 1
 #define KR_SERVE_MIX_ATTENTION 0
 #define KR_SERVE_MIX_LATENT 1
+#define KR_SERVE_MIX_RETENTION 2       /* S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t; k scaled by dim^(-1/2) after the rotation; o / rms(o) per head, times silu(W_g h) */
+#define KR_SERVE_MIX_MLSTM 3           /* exponential input gate and sigmoid forget gate in log space with a running maximum m (m_0 = 0), normaliser state n;
+                                        * q scaled by dim^(-1/2); o = S^T q / (max(|n.q|, exp(-m)) + 1e-6); o / rms(o) per head, times a weight, times sigmoid(W_g h) */
 #define KR_SERVE_QKNORM_NONE 0
 #define KR_SERVE_QKNORM_AFTER_ROT 1    /* no weight, after the rotation */
 #define KR_SERVE_QKNORM_WEIGHTED 2     /* times a weight [dim] shared by the heads (tensors q_norm, k_norm), before the rotation */
+#define KR_SERVE_QKNORM_WHOLE 3        /* one root mean square over ALL heads of q (of k), weights [heads * dim] / [kv_heads * dim], before the rotation */
+#define KR_SERVE_RBIAS_NONE 0
+#define KR_SERVE_RBIAS_LOGIT 1         /* logits + bias before the scores */
+#define KR_SERVE_RBIAS_CHOICE 2        /* scores + bias decide groups and experts; the weights are the scores without it */
+#define KR_SERVE_RSCORE_SOFTMAX 0
+#define KR_SERVE_RSCORE_SIGMOID 1
+#define KR_SERVE_GSCORE_MAX 0
+#define KR_SERVE_GSCORE_TOP2 1
+#define KR_SERVE_OGATE_NONE 0
+#define KR_SERVE_OGATE_HEAD_SIGMOID 1  /* one number per head: tensor out_gate [heads, width] */
 #define KR_SERVE_SINK_NONE 0
 #define KR_SERVE_SINK_TENSOR 1         /* learned score per head */
 #define KR_SERVE_SINK_ZERO 2           /* score 0: one added to the denominator */
@@ -436,9 +470,13 @@ enum { KR_SV_EMBED = 0, KR_SV_FINAL_NORM_W, KR_SV_FINAL_NORM_B, KR_SV_HEAD, KR_S
        KR_SV_NORM2_W, KR_SV_NORM2_B, KR_SV_POST1_W, KR_SV_POST1_B, KR_SV_POST2_W, KR_SV_POST2_B,
        KR_SV_Q_NORM, KR_SV_K_NORM, KR_SV_VMIX, KR_SV_ROUTER_BIAS,
        KR_SV_DQ, KR_SV_DQ_NORM, KR_SV_UQ, KR_SV_DKV, KR_SV_DKV_NORM, KR_SV_UK, KR_SV_UV,     /* latent mixer */
+       KR_SV_Q_BIAS, KR_SV_K_BIAS, KR_SV_O_BIAS,
+       KR_SV_OUT_GATE,                 /* attention: [heads, width]; recurrent mixers: [heads * vdim, width] */
+       KR_SV_CANON, KR_SV_RES_GATE1, KR_SV_RES_GATE1_B, KR_SV_RES_GATE2, KR_SV_RES_GATE2_B,
+       KR_SV_LIN_NORM, KR_SV_LIN_DECAY /* [heads] f32, retention */, KR_SV_IGATE, KR_SV_IGATE_B, KR_SV_FGATE, KR_SV_FGATE_B,     /* recurrent mixers */
        KR_SV_N_ROLES };
 /* layout version of kr_serve_config / kr_serve_layer: a caller built against another one must not use the library */
-#define KR_SERVE_ABI 2
+#define KR_SERVE_ABI 3
 int kr_serve_abi(void);
 int kr_serve_create(int device_ordinal, const kr_serve_config* cfg, const kr_serve_layer* layers, kr_serve** out);
 void kr_serve_destroy(kr_serve* s);

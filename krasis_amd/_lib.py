@@ -48,7 +48,8 @@ class ModelConfigC(C.Structure):
 class ServeConfigC(C.Structure):
     _fields_ = [("vocab", C.c_int), ("width", C.c_int), ("n_layers", C.c_int), ("dtype", C.c_int), ("norm_kind", C.c_int), ("norm_eps", C.c_float),
                 ("max_slots", C.c_int), ("page_tokens", C.c_int), ("pool_tokens", C.c_int),
-                ("block_kind", C.c_int), ("pre_norm", C.c_int), ("post_norm", C.c_int), ("norm_bias", C.c_int), ("residual_mult", C.c_float)]
+                ("block_kind", C.c_int), ("pre_norm", C.c_int), ("post_norm", C.c_int), ("norm_bias", C.c_int), ("residual_mult", C.c_float),
+                ("norm_groups", C.c_int), ("embed_scale", C.c_float), ("canon_taps", C.c_int), ("res_gate", C.c_int)]
 
 
 class ServeLayerC(C.Structure):
@@ -58,10 +59,12 @@ class ServeLayerC(C.Structure):
                 ("top", C.c_int), ("groups", C.c_int), ("keep", C.c_int), ("renorm", C.c_int), ("expert_ff", C.c_int), ("expert_act", C.c_int),
                 ("expert_limit", C.c_float), ("expert_alpha", C.c_float), ("shared_ff", C.c_int), ("shared_limit", C.c_float),
                 ("mixer_kind", C.c_int), ("q_rank", C.c_int), ("kv_rank", C.c_int), ("rot_scaling", C.c_int), ("rot_original", C.c_double), ("rot_fast", C.c_double),
-                ("rot_slow", C.c_double), ("chunk", C.c_int), ("dist_bias", C.c_int), ("dist_bias_exp", C.c_float), ("v_mix", C.c_int), ("router_bias", C.c_int)]
+                ("rot_slow", C.c_double), ("chunk", C.c_int), ("dist_bias", C.c_int), ("dist_bias_exp", C.c_float), ("v_mix", C.c_int), ("router_bias", C.c_int),
+                ("proj_bias", C.c_int), ("v_from_k", C.c_int), ("softcap", C.c_float), ("out_gate", C.c_int), ("gate_cap", C.c_float), ("lin_norm_weight", C.c_int),
+                ("router_score", C.c_int), ("group_score", C.c_int)]
 
 
-SERVE_ABI = 2      # layout version of the two structures above (KR_SERVE_ABI in include/krasis_hip.h)
+SERVE_ABI = 3      # layout version of the two structures above (KR_SERVE_ABI in include/krasis_hip.h)
 
 
 _lib = None

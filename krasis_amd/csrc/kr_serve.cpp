@@ -25,8 +25,15 @@ struct SvLayer {
     // [kv_rank, dim] (W_uk of the head transposed: it multiplies the QUERY) and uv [vdim, kv_rank].
     DevBuf norm_w, norm_b, norm2_w, norm2_b, post1_w, post1_b, post2_w, post2_b, hw, o, sink, down, egu, edown, sdown, kpool, vpool;
     DevBuf q_norm, k_norm, vmix, router_b, slopes, dq_norm, dkv_norm, uq, ukT, uv;
-    int rope_id = 0, n_qkv = 0, off_router = 0, n_router = 0, off_gu = 0, n_gu = 0, n_h = 0;
+    // biases of q / k / o; the input convolution's taps and its per-slot rows; the residual gates (the mixer's is a matrix of its own: it multiplies the
+    // un-convolved input; the feed-forward's is the last row block of hw); recurrent mixers: output norm weight, decays, gate biases, per-slot state
+    DevBuf q_bias, k_bias, o_bias, canon, canon_state, rg1, rg1_b, rg2_b, lin_norm, decay, i_bias, f_bias, lin_state, lin_nm;
+    size_t lin_state_stride = 0, lin_nm_stride = 0;
+    // row blocks of hw: mixer [q | k | v | out gate | i | f] (n_qkv rows in all), then [router | gate | up | residual gate of the feed-forward]
+    int rope_id = 0, n_qkv = 0, off_ogate = 0, off_if = 0, off_router = 0, n_router = 0, off_gu = 0, n_gu = 0, off_rg2 = 0, n_h = 0;
     bool latent() const { return d.mixer_kind == KR_SERVE_MIX_LATENT; }
+    bool recurrent() const { return d.mixer_kind == KR_SERVE_MIX_RETENTION || d.mixer_kind == KR_SERVE_MIX_MLSTM; }
+    bool has_cache() const { return !recurrent() && d.kv_from < 0; }
     int att_heads_kv() const { return latent() ? 1 : d.kv_heads; }
     int att_dim() const { return latent() ? d.kv_rank + d.rot_dims : d.dim; }       // key row of the attention kernels
     int att_vdim() const { return latent() ? d.kv_rank : d.vdim; }
@@ -56,6 +63,7 @@ struct kr_serve {
     std::vector<int> h_table;
     // step scratch
     DevBuf meta, x, h, qkv, att, mix, gu, y, rows, ffout, ids, wts, rz, moe_i, hw, logits, amax, part_ml, part_acc;
+    DevBuf h32, hc, rg, qk_rms, lin_o;                   // f32 copy of the mixer's normed input, its convolved form, residual gate logits, whole-row q / k statistics, recurrent outputs
     DevBuf v_first;                                      // [T, kv_heads * vdim] f32: the values of the first value-mixing layer
     DevBuf lq_c, lq_2, lq_n, lq_e, att2, head_i;         // latent mixer: query latent, W_uq output, plain query parts, folded queries, per-head values, head row tables
     void* h_meta = nullptr; size_t h_meta_bytes = 0;     // pinned staging of the per-step arrays
@@ -111,14 +119,26 @@ int check_layer(const kr_serve_config& c, const kr_serve_layer* all, int i) {
     if (d.heads < 1 || d.kv_heads < 1 || d.heads % d.kv_heads) return kr_fail(KR_ERR_VALUE, "layer %d: heads %d / kv_heads %d", i, d.heads, d.kv_heads);
     if (d.dim < 1 || d.vdim < 1 || d.vdim > 512 || d.dim > 512) return kr_fail(KR_ERR_VALUE, "layer %d: head sizes %d / %d (at most 512)", i, d.dim, d.vdim);
     const bool lat = d.mixer_kind == KR_SERVE_MIX_LATENT;
-    if (d.mixer_kind != KR_SERVE_MIX_ATTENTION && !lat) return kr_fail(KR_ERR_VALUE, "layer %d: mixer kind %d", i, d.mixer_kind);
+    const bool rec = d.mixer_kind == KR_SERVE_MIX_RETENTION || d.mixer_kind == KR_SERVE_MIX_MLSTM;
+    if (d.mixer_kind != KR_SERVE_MIX_ATTENTION && !lat && !rec) return kr_fail(KR_ERR_VALUE, "layer %d: mixer kind %d", i, d.mixer_kind);
+    if (rec) {
+        if (d.kv_heads != d.heads || d.dim > 256) return kr_fail(KR_ERR_VALUE, "layer %d: a recurrent mixer has one key / value head per query head and dim <= 256", i);
+        if (d.kv_from >= 0 || d.v_mix || d.qk_unit_norm || d.window || d.chunk || d.has_sink || d.dist_bias || d.proj_bias || d.v_from_k || d.out_gate || d.softcap != 0.0f)
+            return kr_fail(KR_ERR_VALUE, "layer %d: an attention-only mechanism is switched on for a recurrent mixer", i);
+        if (d.rot_dims && (d.rot_interleaved || d.mixer_kind != KR_SERVE_MIX_RETENTION)) return kr_fail(KR_ERR_VALUE, "layer %d: recurrent mixers rotate half-split pairs, retention only", i);
+    } else if (d.gate_cap != 0.0f || d.lin_norm_weight) return kr_fail(KR_ERR_VALUE, "layer %d: gate_cap / lin_norm_weight belong to recurrent mixers", i);
+    if (d.v_from_k && (lat || d.vdim != d.dim || d.v_mix || d.kv_from >= 0)) return kr_fail(KR_ERR_VALUE, "layer %d: values that are the keys need vdim == dim, a cache of their own and no value mixing", i);
+    if ((d.proj_bias || d.out_gate) && lat) return kr_fail(KR_ERR_VALUE, "layer %d: a latent mixer has no projection biases / output gate", i);
+    if (d.out_gate < 0 || d.out_gate > KR_SERVE_OGATE_HEAD_SIGMOID || d.softcap < 0.0f || d.router_bias < 0 || d.router_bias > KR_SERVE_RBIAS_CHOICE || d.router_score < 0 ||
+        d.router_score > KR_SERVE_RSCORE_SIGMOID || d.group_score < 0 || d.group_score > KR_SERVE_GSCORE_TOP2)
+        return kr_fail(KR_ERR_VALUE, "layer %d: output gate %d / softcap %g / router bias %d / score %d / group score %d", i, d.out_gate, (double)d.softcap, d.router_bias, d.router_score, d.group_score);
     if (d.rot_dims < 0 || (!lat && d.rot_dims > d.dim) || (d.rot_dims & 1)) return kr_fail(KR_ERR_VALUE, "layer %d: rot_dims %d of %d", i, d.rot_dims, d.dim);
     if (d.rot_dims && (!(d.rot_base > 0.0) || !(d.rot_factor > 0.0))) return kr_fail(KR_ERR_VALUE, "layer %d: rotation base / factor", i);
     if (d.rot_scaling != KR_SERVE_ROT_LINEAR && d.rot_scaling != KR_SERVE_ROT_BY_PARTS) return kr_fail(KR_ERR_VALUE, "layer %d: rotation scaling %d", i, d.rot_scaling);
     if (d.rot_dims && d.rot_scaling == KR_SERVE_ROT_BY_PARTS && (!(d.rot_original > 0.0) || !(d.rot_fast > 0.0) || !(d.rot_slow > 0.0) || !(d.rot_base > 1.0)))
         return kr_fail(KR_ERR_VALUE, "layer %d: by-parts rotation scaling needs original, fast, slow > 0 and base > 1", i);
     if (d.window < 0 || d.chunk < 0 || (d.window > 0 && d.chunk > 0)) return kr_fail(KR_ERR_VALUE, "layer %d: window %d / chunk %d", i, d.window, d.chunk);
-    if (d.qk_unit_norm < 0 || d.qk_unit_norm > KR_SERVE_QKNORM_WEIGHTED || d.has_sink < 0 || d.has_sink > KR_SERVE_SINK_ZERO || d.v_mix < 0 || d.v_mix > KR_SERVE_VMIX_BLEND)
+    if (d.qk_unit_norm < 0 || d.qk_unit_norm > KR_SERVE_QKNORM_WHOLE || d.has_sink < 0 || d.has_sink > KR_SERVE_SINK_ZERO || d.v_mix < 0 || d.v_mix > KR_SERVE_VMIX_BLEND)
         return kr_fail(KR_ERR_VALUE, "layer %d: qk norm %d / sink %d / value mixing %d", i, d.qk_unit_norm, d.has_sink, d.v_mix);
     if (lat) {
         if (d.q_rank < 1 || d.kv_rank < 1 || d.kv_rank > 512 || d.kv_rank + d.rot_dims > 1024) return kr_fail(KR_ERR_VALUE, "layer %d: latent sizes %d / %d", i, d.q_rank, d.kv_rank);
@@ -170,6 +190,10 @@ int kr_serve_create(int device_ordinal, const kr_serve_config* cfg, const kr_ser
     if (cfg->max_slots < 1 || cfg->page_tokens < 1 || cfg->pool_tokens < cfg->page_tokens) return kr_fail(KR_ERR_VALUE, "slots / pages");
     if (cfg->block_kind != KR_SERVE_BLOCK_PARALLEL && cfg->block_kind != KR_SERVE_BLOCK_SEQUENTIAL) return kr_fail(KR_ERR_VALUE, "block kind %d", cfg->block_kind);
     if (cfg->post_norm && cfg->block_kind != KR_SERVE_BLOCK_SEQUENTIAL) return kr_fail(KR_ERR_VALUE, "norms on sublayer outputs need a sequential block");
+    if (cfg->norm_groups < 0 || (cfg->norm_groups > 1 && cfg->width % cfg->norm_groups)) return kr_fail(KR_ERR_VALUE, "norm groups %d of width %d", cfg->norm_groups, cfg->width);
+    if (cfg->canon_taps < 0 || cfg->canon_taps == 1 || cfg->canon_taps > 64) return kr_fail(KR_ERR_VALUE, "input convolution of %d taps", cfg->canon_taps);
+    if ((cfg->canon_taps || cfg->res_gate) && !(cfg->block_kind == KR_SERVE_BLOCK_SEQUENTIAL && cfg->pre_norm && !cfg->post_norm))
+        return kr_fail(KR_ERR_VALUE, "input convolution / gated residual need a sequential pre-normed block without output norms");
     for (int i = 0; i < cfg->n_layers; i++) { const int rc = check_layer(*cfg, layers, i); if (rc) return rc; }
     int n_dev = 0;
     if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev <= device_ordinal) return kr_fail(KR_ERR_HIP, "no HIP device %d (the serving store has no CPU path)", device_ordinal);
@@ -187,10 +211,15 @@ int kr_serve_create(int device_ordinal, const kr_serve_config* cfg, const kr_ser
         SvLayer& l = s->L[i]; l.d = layers[i];
         const kr_serve_layer& d = l.d;
         l.have.assign(KR_SV_N_ROLES, 0);
-        l.n_qkv = l.latent() ? d.q_rank + d.kv_rank + d.rot_dims : d.heads * d.dim + (d.kv_from < 0 ? d.kv_heads * (d.dim + d.vdim) : 0);
+        l.n_qkv = l.latent() ? d.q_rank + d.kv_rank + d.rot_dims : d.heads * d.dim + (d.kv_from < 0 ? d.kv_heads * (d.dim + (d.v_from_k ? 0 : d.vdim)) : 0);
+        l.off_ogate = l.n_qkv;
+        if (l.recurrent()) l.n_qkv += d.heads * d.vdim; else if (d.out_gate) l.n_qkv += d.heads;
+        l.off_if = l.n_qkv;
+        if (d.mixer_kind == KR_SERVE_MIX_MLSTM) l.n_qkv += 2 * d.heads;
         l.n_router = d.mlp_kind == KR_SERVE_MLP_MOE ? d.experts * (s->f32 ? 1 : 2) : 0;
         l.n_gu = d.mlp_kind == KR_SERVE_MLP_DENSE ? 2 * d.ff : (d.mlp_kind == KR_SERVE_MLP_MOE ? 2 * d.shared_ff : 0);
-        l.off_router = l.n_qkv; l.off_gu = l.off_router + l.n_router; l.n_h = l.off_gu + l.n_gu;
+        l.off_router = l.n_qkv; l.off_gu = l.off_router + l.n_router; l.off_rg2 = l.off_gu + l.n_gu;
+        l.n_h = l.off_rg2 + ((cfg->res_gate && d.mlp_kind != KR_SERVE_MLP_NONE) ? cfg->width : 0);
         if (d.mlp_kind == KR_SERVE_MLP_MOE) { l.eg.assign(d.experts, 0); l.eu.assign(d.experts, 0); l.ed.assign(d.experts, 0); }
         if (d.rot_dims > 0) {
             const bool parts = d.rot_scaling == KR_SERVE_ROT_BY_PARTS;
@@ -231,7 +260,18 @@ int kr_serve_create(int device_ordinal, const kr_serve_config* cfg, const kr_ser
         if (d.has_sink == KR_SERVE_SINK_ZERO) {
             if (l.sink.ensure((size_t)d.heads * 4) || hipMemset(l.sink.p, 0, (size_t)d.heads * 4) != hipSuccess) { kr_serve_destroy(s); return kr_fail(KR_ERR_HIP, "sink"); }
         }
-        if (d.kv_from < 0) {
+        if (cfg->canon_taps > 1) {
+            const size_t b = (size_t)cfg->max_slots * (cfg->canon_taps - 1) * cfg->width * 4;
+            if (l.canon_state.ensure(b) || hipMemset(l.canon_state.p, 0, b) != hipSuccess) { kr_serve_destroy(s); return kr_fail(KR_ERR_HIP, "input convolution state"); }
+        }
+        if (l.recurrent()) {
+            l.lin_state_stride = (size_t)d.heads * d.vdim * d.dim; l.lin_nm_stride = (size_t)d.heads * ((d.vdim + 15) / 16) * (d.dim + 4);
+            const size_t sb = l.lin_state_stride * cfg->max_slots * 4, nb = l.lin_nm_stride * cfg->max_slots * 4;
+            if (l.lin_state.ensure(sb) || l.lin_nm.ensure(nb) || hipMemset(l.lin_state.p, 0, sb) != hipSuccess || hipMemset(l.lin_nm.p, 0, nb) != hipSuccess) {
+                kr_serve_destroy(s); return kr_fail(KR_ERR_HIP, "recurrent state of %zu bytes", sb + nb);
+            }
+        }
+        if (l.has_cache()) {
             const size_t rows = (size_t)s->n_pages * cfg->page_tokens;
             const size_t kb = rows * l.att_heads_kv() * l.att_dim() * s->esz, vb = l.latent() ? 0 : rows * d.kv_heads * d.vdim * s->esz;     // a latent's values are its key rows
             if (l.kpool.ensure(kb) || (vb && l.vpool.ensure(vb))) { kr_serve_destroy(s); return kr_fail(KR_ERR_HIP, "cache pool of %zu bytes", kb + vb); }
@@ -278,8 +318,40 @@ int kr_serve_set_tensor(kr_serve* s, int layer, int role, int index, const void*
     const bool lat = l.latent();
     if (lat && (role == KR_SV_Q || role == KR_SV_K || role == KR_SV_V)) return kr_fail(KR_ERR_VALUE, "layer %d has a latent mixer", layer);
     if (!lat && role >= KR_SV_DQ && role <= KR_SV_UV) return kr_fail(KR_ERR_VALUE, "layer %d has no latent mixer", layer);
+    const bool rec = l.recurrent();
     int rc = KR_OK;
     switch (role) {
+    case KR_SV_Q_BIAS: case KR_SV_K_BIAS: case KR_SV_O_BIAS:
+        if (!d.proj_bias) return kr_fail(KR_ERR_VALUE, "layer %d has no projection biases", layer);
+        SHAPE(1, role == KR_SV_Q_BIAS ? nq : role == KR_SV_K_BIAS ? nk : W);
+        rc = upload(s, role == KR_SV_Q_BIAS ? l.q_bias : role == KR_SV_K_BIAS ? l.k_bias : l.o_bias, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_OUT_GATE:
+        if (!rec && !d.out_gate) return kr_fail(KR_ERR_VALUE, "layer %d has no output gate", layer);
+        SHAPE(rec ? d.heads * d.vdim : d.heads, W); rc = upload(s, l.hw, (size_t)l.n_h * W, (size_t)l.off_ogate * W, host, src_dtype, n, false); break;
+    case KR_SV_IGATE: case KR_SV_FGATE:
+        if (d.mixer_kind != KR_SERVE_MIX_MLSTM) return kr_fail(KR_ERR_VALUE, "layer %d has no input / forget gates", layer);
+        SHAPE(d.heads, W); rc = upload(s, l.hw, (size_t)l.n_h * W, ((size_t)l.off_if + (role == KR_SV_FGATE ? d.heads : 0)) * W, host, src_dtype, n, false); break;
+    case KR_SV_IGATE_B: case KR_SV_FGATE_B:
+        if (d.mixer_kind != KR_SERVE_MIX_MLSTM) return kr_fail(KR_ERR_VALUE, "layer %d has no input / forget gates", layer);
+        SHAPE(1, d.heads); rc = upload(s, role == KR_SV_IGATE_B ? l.i_bias : l.f_bias, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_LIN_NORM:
+        if (!rec || !d.lin_norm_weight) return kr_fail(KR_ERR_VALUE, "layer %d has no weight on its mixer's output norm", layer);
+        SHAPE(1, d.heads * d.vdim); rc = upload(s, l.lin_norm, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_LIN_DECAY:
+        if (d.mixer_kind != KR_SERVE_MIX_RETENTION) return kr_fail(KR_ERR_VALUE, "layer %d is no retention layer", layer);
+        SHAPE(1, d.heads); rc = upload(s, l.decay, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_CANON:
+        if (s->c.canon_taps < 2) return kr_fail(KR_ERR_VALUE, "the design has no input convolution");
+        SHAPE(W, s->c.canon_taps); rc = upload(s, l.canon, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_RES_GATE1: case KR_SV_RES_GATE2:
+        if (!s->c.res_gate || (role == KR_SV_RES_GATE2 && d.mlp_kind == KR_SERVE_MLP_NONE)) return kr_fail(KR_ERR_VALUE, "layer %d has no such residual gate", layer);
+        SHAPE(W, W);
+        if (role == KR_SV_RES_GATE1) rc = upload(s, l.rg1, n, 0, host, src_dtype, n, false);
+        else rc = upload(s, l.hw, (size_t)l.n_h * W, (size_t)l.off_rg2 * W, host, src_dtype, n, false);
+        break;
+    case KR_SV_RES_GATE1_B: case KR_SV_RES_GATE2_B:
+        if (!s->c.res_gate || (role == KR_SV_RES_GATE2_B && d.mlp_kind == KR_SERVE_MLP_NONE)) return kr_fail(KR_ERR_VALUE, "layer %d has no such residual gate", layer);
+        SHAPE(1, W); rc = upload(s, role == KR_SV_RES_GATE1_B ? l.rg1_b : l.rg2_b, n, 0, host, src_dtype, n, true); break;
     case KR_SV_NORM2_W: SHAPE(1, W); rc = upload(s, l.norm2_w, n, 0, host, src_dtype, n, true); break;
     case KR_SV_NORM2_B: SHAPE(1, W); rc = upload(s, l.norm2_b, n, 0, host, src_dtype, n, true); break;
     case KR_SV_POST1_W: SHAPE(1, W); rc = upload(s, l.post1_w, n, 0, host, src_dtype, n, true); break;
@@ -287,8 +359,8 @@ int kr_serve_set_tensor(kr_serve* s, int layer, int role, int index, const void*
     case KR_SV_POST2_W: SHAPE(1, W); rc = upload(s, l.post2_w, n, 0, host, src_dtype, n, true); break;
     case KR_SV_POST2_B: SHAPE(1, W); rc = upload(s, l.post2_b, n, 0, host, src_dtype, n, true); break;
     case KR_SV_Q_NORM: case KR_SV_K_NORM:
-        if (d.qk_unit_norm != KR_SERVE_QKNORM_WEIGHTED) return kr_fail(KR_ERR_VALUE, "layer %d has no weighted q / k norm", layer);
-        SHAPE(1, d.dim); rc = upload(s, role == KR_SV_Q_NORM ? l.q_norm : l.k_norm, n, 0, host, src_dtype, n, true); break;
+        if (d.qk_unit_norm != KR_SERVE_QKNORM_WEIGHTED && d.qk_unit_norm != KR_SERVE_QKNORM_WHOLE) return kr_fail(KR_ERR_VALUE, "layer %d has no weighted q / k norm", layer);
+        SHAPE(1, d.qk_unit_norm == KR_SERVE_QKNORM_WHOLE ? (role == KR_SV_Q_NORM ? nq : nk) : d.dim); rc = upload(s, role == KR_SV_Q_NORM ? l.q_norm : l.k_norm, n, 0, host, src_dtype, n, true); break;
     case KR_SV_VMIX: if (d.v_mix != KR_SERVE_VMIX_BLEND) return kr_fail(KR_ERR_VALUE, "layer %d blends no values", layer);
         SHAPE(1, 1); rc = upload(s, l.vmix, n, 0, host, src_dtype, n, true); break;
     case KR_SV_ROUTER_BIAS: if (!moe || !d.router_bias) return kr_fail(KR_ERR_VALUE, "layer %d has no router bias", layer);
@@ -315,7 +387,7 @@ int kr_serve_set_tensor(kr_serve* s, int layer, int role, int index, const void*
     case KR_SV_Q: SHAPE(nq, W); rc = upload(s, l.hw, (size_t)l.n_h * W, 0, host, src_dtype, n, false); break;
     case KR_SV_K: if (d.kv_from >= 0) return kr_fail(KR_ERR_VALUE, "layer %d borrows its keys", layer);
         SHAPE(nk, W); rc = upload(s, l.hw, (size_t)l.n_h * W, (size_t)nq * W, host, src_dtype, n, false); break;
-    case KR_SV_V: if (d.kv_from >= 0) return kr_fail(KR_ERR_VALUE, "layer %d borrows its values", layer);
+    case KR_SV_V: if (d.kv_from >= 0 || d.v_from_k) return kr_fail(KR_ERR_VALUE, "layer %d has no value projection", layer);
         SHAPE(nv, W); rc = upload(s, l.hw, (size_t)l.n_h * W, (size_t)(nq + nk) * W, host, src_dtype, n, false); break;
     case KR_SV_O: SHAPE(W, d.heads * d.vdim); rc = upload(s, l.o, n, 0, host, src_dtype, n, false); break;
     case KR_SV_SINK: if (d.has_sink != KR_SERVE_SINK_TENSOR) return kr_fail(KR_ERR_VALUE, "layer %d has no sink tensor", layer);
@@ -389,6 +461,26 @@ int kr_serve_fill_synthetic(kr_serve* s, uint64_t seed, float amp) {
         if (s->c.post_norm) bad |= vec(l.post1_w, W, true) | vec(l.post2_w, W, true) | (nb ? vec(l.post1_b, W, false) | vec(l.post2_b, W, false) : 0);
         if (d.has_sink == KR_SERVE_SINK_TENSOR) bad |= vec(l.sink, d.heads, false);
         if (d.qk_unit_norm == KR_SERVE_QKNORM_WEIGHTED) bad |= vec(l.q_norm, d.dim, true) | vec(l.k_norm, d.dim, true);
+        if (d.qk_unit_norm == KR_SERVE_QKNORM_WHOLE) bad |= vec(l.q_norm, (size_t)d.heads * d.dim, true) | vec(l.k_norm, (size_t)d.kv_heads * d.dim, true);
+        if (d.proj_bias) bad |= vec(l.q_bias, (size_t)d.heads * d.dim, false) | vec(l.k_bias, (size_t)d.kv_heads * d.dim, false) | vec(l.o_bias, W, false);
+        if (s->c.canon_taps > 1) {           // taps of 1 / (2 taps): the convolved input stays at the input's scale
+            bad |= vec(l.canon, (size_t)W * s->c.canon_taps, true);
+            if (!bad) kr_sv_fill_uniform(l.canon.p, true, (size_t)W * s->c.canon_taps, ++k, 0.5f / (float)s->c.canon_taps, s->st);
+        }
+        if (s->c.res_gate) {
+            bad |= mat(l.rg1, (size_t)W * W, W) | vec(l.rg1_b, W, false);
+            if (d.mlp_kind != KR_SERVE_MLP_NONE) bad |= vec(l.rg2_b, W, false);
+        }
+        if (l.recurrent()) {
+            if (d.lin_norm_weight) bad |= vec(l.lin_norm, (size_t)d.heads * d.vdim, true);
+            if (d.mixer_kind == KR_SERVE_MIX_MLSTM) bad |= vec(l.i_bias, d.heads, false) | vec(l.f_bias, d.heads, true);
+            else {
+                std::vector<float> dc(d.heads);
+                for (int h = 0; h < d.heads; h++) dc[h] = 1.0f - std::exp2(-5.0f - (float)(h % 8));
+                bad |= vec(l.decay, d.heads, true);
+                if (!bad) bad |= hipMemcpy(l.decay.p, dc.data(), dc.size() * 4, hipMemcpyHostToDevice) != hipSuccess;
+            }
+        }
         if (d.v_mix == KR_SERVE_VMIX_BLEND) { bad |= vec(l.vmix, 1, true); const float half = 0.5f; bad |= hipMemcpy(l.vmix.p, &half, 4, hipMemcpyHostToDevice) != hipSuccess; }
         if (l.latent()) {
             bad |= vec(l.dq_norm, d.q_rank, true) | vec(l.dkv_norm, d.kv_rank, true) | mat(l.uq, (size_t)d.heads * (d.dim + d.rot_dims) * d.q_rank, d.q_rank) |
@@ -425,9 +517,16 @@ int kr_serve_finalize(kr_serve* s) {
         if (l.latent()) for (int r : {KR_SV_DQ, KR_SV_DQ_NORM, KR_SV_UQ, KR_SV_DKV, KR_SV_DKV_NORM, KR_SV_UK, KR_SV_UV}) need.push_back(r);
         else {
             need.push_back(KR_SV_Q);
-            if (d.kv_from < 0) { need.push_back(KR_SV_K); need.push_back(KR_SV_V); }
+            if (d.kv_from < 0) { need.push_back(KR_SV_K); if (!d.v_from_k) need.push_back(KR_SV_V); }
         }
-        if (d.qk_unit_norm == KR_SERVE_QKNORM_WEIGHTED) { need.push_back(KR_SV_Q_NORM); if (d.kv_from < 0) need.push_back(KR_SV_K_NORM); }
+        if (d.qk_unit_norm == KR_SERVE_QKNORM_WEIGHTED || d.qk_unit_norm == KR_SERVE_QKNORM_WHOLE) { need.push_back(KR_SV_Q_NORM); if (d.kv_from < 0) need.push_back(KR_SV_K_NORM); }
+        if (d.proj_bias) { need.push_back(KR_SV_Q_BIAS); need.push_back(KR_SV_O_BIAS); if (d.kv_from < 0) need.push_back(KR_SV_K_BIAS); }
+        if (d.out_gate || l.recurrent()) need.push_back(KR_SV_OUT_GATE);
+        if (l.recurrent() && d.lin_norm_weight) need.push_back(KR_SV_LIN_NORM);
+        if (d.mixer_kind == KR_SERVE_MIX_RETENTION) need.push_back(KR_SV_LIN_DECAY);
+        if (d.mixer_kind == KR_SERVE_MIX_MLSTM) for (int r : {KR_SV_IGATE, KR_SV_IGATE_B, KR_SV_FGATE, KR_SV_FGATE_B}) need.push_back(r);
+        if (s->c.canon_taps > 1) need.push_back(KR_SV_CANON);
+        if (s->c.res_gate) { need.push_back(KR_SV_RES_GATE1); need.push_back(KR_SV_RES_GATE1_B); if (has_ff) { need.push_back(KR_SV_RES_GATE2); need.push_back(KR_SV_RES_GATE2_B); } }
         if (d.v_mix == KR_SERVE_VMIX_BLEND) need.push_back(KR_SV_VMIX);
         if (d.has_sink == KR_SERVE_SINK_TENSOR) need.push_back(KR_SV_SINK);
         if (d.mlp_kind == KR_SERVE_MLP_DENSE) { need.push_back(KR_SV_GATE); need.push_back(KR_SV_UP); need.push_back(KR_SV_DOWN); }
@@ -505,7 +604,7 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
     for (int i = 0; i < n_want; i++) if (want_rows[i] < 0 || want_rows[i] >= T) return kr_fail(KR_ERR_VALUE, "wanted row %d of %d", want_rows[i], T);
     if (need_pages > (int)s->free_pages.size()) return kr_fail(KR_ERR_STATE, "cache pool exhausted: %d pages needed, %zu free", need_pages, s->free_pages.size());
     // ---- per-step arrays: tokens | slot | pos | want | page table
-    const size_t n_meta = (size_t)3 * T + n_want;
+    const size_t n_meta = (size_t)3 * T + n_want + 2 * (size_t)n_entries + 1;      // ... | first row of every entry and the end | slot of every entry
     const size_t meta_bytes = (n_meta + s->h_table.size()) * 4;
     if (meta_bytes > s->h_meta_bytes) {
         if (s->h_meta) (void)hipHostFree(s->h_meta);
@@ -514,19 +613,22 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         s->h_meta_bytes = meta_bytes * 2;
     }
     int* hm = (int*)s->h_meta;
-    int* h_tok = hm; int* h_slot = hm + T; int* h_pos = hm + 2 * T; int* h_want = hm + 3 * T; int* h_tab = hm + n_meta;
+    int* h_tok = hm; int* h_slot = hm + T; int* h_pos = hm + 2 * T; int* h_want = hm + 3 * T; int* h_eoff = h_want + n_want; int* h_eslot = h_eoff + n_entries + 1;
+    int* h_tab = hm + n_meta;
     int max_pos = 0;
     {
         int t = 0;
         for (int e = 0; e < n_entries; e++) {
             SvSlot& q = s->slots[slots[e]];
             max_pos = std::max(max_pos, q.len + counts[e] - 1);
+            h_eoff[e] = t; h_eslot[e] = slots[e];
             const int np = (q.len + counts[e] + PT - 1) / PT;
             while ((int)q.pages.size() < np) { q.pages.push_back(s->free_pages.back()); s->free_pages.pop_back(); }
             for (int i = 0; i < counts[e]; i++, t++) { h_tok[t] = tokens[t]; h_slot[t] = slots[e]; h_pos[t] = q.len + i; }
             for (size_t p = 0; p < q.pages.size(); p++) s->h_table[(size_t)slots[e] * s->n_pages + p] = q.pages[p];
             q.len += counts[e];
         }
+        h_eoff[n_entries] = t;
         for (int i = 0; i < n_want; i++) h_want[i] = want_rows[i];
         std::memcpy(h_tab, s->h_table.data(), s->h_table.size() * 4);
     }
@@ -534,13 +636,16 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
     hipStream_t st = s->st;
     KR_HIP(hipMemcpyAsync(s->meta.p, hm, meta_bytes, hipMemcpyHostToDevice, st));
     const int* d_tok = (const int*)s->meta.p; const int* d_slot = d_tok + T; const int* d_pos = d_tok + 2 * T; const int* d_want = d_tok + 3 * T;
+    const int* d_eoff = d_want + n_want; const int* d_eslot = d_eoff + n_entries + 1;
     const int* d_tab = d_tok + n_meta;
     // ---- scratch sized for this step
     const bool seq = c.block_kind == KR_SERVE_BLOCK_SEQUENTIAL;
     size_t max_qkv = 0, max_att = 0, max_gu = 0, max_y = 0, max_rows = 0, max_pairs = 0, max_vf = 0; int max_E = 1;
-    size_t lq_c = 0, lq_2 = 0, lq_n = 0, lq_e = 0, att2 = 0, head_i = 0;
+    size_t lq_c = 0, lq_2 = 0, lq_n = 0, lq_e = 0, att2 = 0, head_i = 0, max_lin = 0; bool whole_norm = false;
     for (const SvLayer& l : s->L) {
         const kr_serve_layer& d = l.d;
+        if (l.recurrent()) max_lin = std::max(max_lin, (size_t)d.heads * d.vdim);
+        if (d.qk_unit_norm == KR_SERVE_QKNORM_WHOLE) whole_norm = true;
         max_qkv = std::max(max_qkv, (size_t)l.n_h); max_att = std::max(max_att, (size_t)d.heads * l.att_vdim());
         if (d.v_mix) max_vf = std::max(max_vf, (size_t)d.kv_heads * d.vdim);
         if (l.latent()) {
@@ -564,11 +669,15 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         (head_i && (s->lq_c.ensure(Ts * lq_c * s->esz) || s->lq_2.ensure(Ts * lq_2 * 4) || s->lq_n.ensure(Ts * lq_n * s->esz) || s->lq_e.ensure(Ts * lq_e * 4) ||
                     s->att2.ensure(Ts * att2 * s->esz) || s->head_i.ensure((2 * Ts * head_i + head_i + 1) * 4))))
         return kr_fail(KR_ERR_HIP, "mixer scratch for %d tokens", T);
+    if ((c.canon_taps > 1 && (s->h32.ensure(Ts * W * 4) || s->hc.ensure(Ts * W * s->esz))) || (c.res_gate && s->rg.ensure(Ts * W * 4)) || (whole_norm && s->qk_rms.ensure(Ts * 2 * 4)) ||
+        (max_lin && s->lin_o.ensure(Ts * max_lin * 4)))
+        return kr_fail(KR_ERR_HIP, "block scratch for %d tokens", T);
     for (SvRope& r : s->ropes) if (r.cs.ensure(Ts * (r.dims / 2) * 8)) return kr_fail(KR_ERR_HIP, "rope table");
     if (s->capture) { if (s->cap.ensure((size_t)c.n_layers * Ts * W * 4)) return kr_fail(KR_ERR_HIP, "capture buffer"); s->cap_T = T; }
     std::vector<int> nsplit(c.n_layers, 1);
     for (int li = 0; li < c.n_layers; li++) {
         const SvLayer& l = s->L[li]; const kr_serve_layer& d = l.d;
+        if (l.recurrent()) continue;
         const int visible = d.window > 0 ? std::min(max_pos + 1, d.window) : (d.chunk > 0 ? std::min(max_pos + 1, d.chunk) : max_pos + 1);
         const int ldk = l.latent() ? l.att_dim() : d.kv_heads * d.dim, ldv = l.latent() ? l.att_dim() : d.kv_heads * d.vdim;
         nsplit[li] = kr_sv_attention_splits(T, d.heads, l.att_heads_kv(), l.att_dim(), l.att_vdim(), ldk, ldv, s->f32, visible);
@@ -581,7 +690,7 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
     float* x = (float*)s->x.p;
     {
         Timer tm(s, 7);
-        kr_sv_embed(s->embed.p, s->f32, d_tok, x, c.pre_norm ? nullptr : s->h.p, T, W, st);     // without input norms the first sublayer reads the embedding row itself
+        kr_sv_embed(s->embed.p, s->f32, d_tok, x, c.pre_norm ? nullptr : s->h.p, T, W, c.embed_scale != 0.0f ? c.embed_scale : 1.0f, st);     // without input norms the first sublayer reads the embedding row itself
     }
     {
         Timer tm(s, 2);
@@ -597,17 +706,36 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
     };
     // the residual sum that ends a sublayer (or, in a parallel block, the layer); `next`: the norm of the sublayer that reads the new x, null with
     // hand_on = the row as it is, or nothing when no sublayer follows
+    const int NG = c.norm_groups > 1 ? c.norm_groups : 1;
+    const bool canon = c.canon_taps > 1;
+    // gate: 0 none, 1 the mixer's (logits in rg, the output projection's bias, and the input convolution's rows of this layer are kept), 2 the feed-forward's
+    // (logits in the last row block of hz).  to_mixer: the handed-on row feeds a mixer (an f32 copy goes along for its input convolution)
+    const SvLayer* res_layer = nullptr; int res_gate_kind = 0; bool res_to_mixer = false;
     auto residual = [&](const float* mixp, const float* dense, const float* shared, const float* rows, const int* pair_pos, int top, const DevBuf* post_w, const DevBuf* post_b,
                         bool hand_on, const DevBuf* next_w, const DevBuf* next_b) {
         Timer tm(s, 6);
         KrSvResidual r{};
+        r.groups = NG;
+        if (res_layer) {
+            const SvLayer& rl = *res_layer;
+            if (mixp && rl.d.proj_bias) r.mix_bias = (const float*)rl.o_bias.p;
+            if (res_gate_kind == 1) {
+                if (c.res_gate) { r.gate = (const float*)s->rg.p; r.ld_gate = W; r.gate_b = (const float*)rl.rg1_b.p; }
+                if (canon) { r.h32_in = (const float*)s->h32.p; r.canon_state = (float*)rl.canon_state.p; r.canon_keep = c.canon_taps - 1; r.slot = d_slot; r.pos = d_pos; }
+            } else if (res_gate_kind == 2 && c.res_gate) { r.gate = (const float*)s->qkv.p + rl.off_rg2; r.ld_gate = rl.n_h; r.gate_b = (const float*)rl.rg2_b.p; }
+        }
+        if (canon && hand_on && res_to_mixer) r.h32_out = (float*)s->h32.p;
         r.x = x; r.mix = mixp; r.dense = dense; r.shared = shared; r.rows = rows; r.pair_pos = pair_pos; r.wts = (const float*)s->wts.p; r.top = top;
         r.post_w = post_w ? (const float*)post_w->p : nullptr; r.post_b = (post_w && c.norm_bias && post_b) ? (const float*)post_b->p : nullptr; r.mult = c.residual_mult;
         r.norm_w = (hand_on && next_w) ? (const float*)next_w->p : nullptr; r.norm_b = (hand_on && next_w && c.norm_bias && next_b) ? (const float*)next_b->p : nullptr;
         r.h_out = hand_on ? s->h.p : nullptr; r.T = T; r.width = W; r.kind = c.norm_kind; r.eps = c.norm_eps;
         kr_sv_residual_norm(r, s->f32, st);
     };
-    if (c.pre_norm) { Timer tm(s, 0); kr_sv_norm(x, nullptr, (const float*)s->L[0].norm_w.p, c.norm_bias ? (const float*)s->L[0].norm_b.p : nullptr, s->h.p, s->f32, T, W, c.norm_eps, c.norm_kind, st); }
+    if (c.pre_norm) {
+        Timer tm(s, 0);
+        kr_sv_norm(x, nullptr, (const float*)s->L[0].norm_w.p, c.norm_bias ? (const float*)s->L[0].norm_b.p : nullptr, s->h.p, s->f32, T, W, c.norm_eps, c.norm_kind, NG,
+                   canon ? (float*)s->h32.p : nullptr, st);
+    }
     int head_rows_for = 0;               // the head row tables in head_i are valid for this head count
     for (int li = 0; li < c.n_layers; li++) {
         SvLayer& l = s->L[li]; const kr_serve_layer& d = l.d;
@@ -616,7 +744,18 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         float* hz = (float*)s->qkv.p;                    // [T, n_h]: q | k | v (or the latents) | router logits | gate | up of this layer
         KrSvGemm g{};
         // a parallel block multiplies its one input by every matrix at once; a sequential block's feed-forward reads the x its mixer leaves
-        g.A = s->h.p; g.lda = W; g.W = l.hw.p; g.C = hz; g.ldc = l.n_h; g.M = T; g.N = seq ? l.n_qkv : l.n_h; g.K = W;
+        const void* mixer_in = s->h.p;
+        if (canon) {       // the mixer reads h + conv(h); the residual gate below reads h itself
+            KrSvCanon cv{}; cv.h32 = (const float*)s->h32.p; cv.w = (const float*)l.canon.p; cv.taps = c.canon_taps; cv.state = (float*)l.canon_state.p;
+            cv.slot = d_slot; cv.pos = d_pos; cv.T = T; cv.width = W; cv.out = s->hc.p;
+            Timer tm(s, 0); kr_sv_canon(cv, s->f32, st);
+            mixer_in = s->hc.p;
+        }
+        if (c.res_gate) {
+            KrSvGemm gg{}; gg.A = s->h.p; gg.lda = W; gg.W = l.rg1.p; gg.C = (float*)s->rg.p; gg.ldc = W; gg.M = T; gg.N = W; gg.K = W;
+            Timer tm(s, 1); kr_sv_gemm(gg, s->f32, st);
+        }
+        g.A = mixer_in; g.lda = W; g.W = l.hw.p; g.C = hz; g.ldc = l.n_h; g.M = T; g.N = seq ? l.n_qkv : l.n_h; g.K = W;
         { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
         const SvLayer& kvl = d.kv_from >= 0 ? s->L[d.kv_from] : l;
         KrSvAttn a{};
@@ -627,12 +766,28 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         a.out = s->att.p;
         a.nsplit = nsplit[li]; a.part_ml = (float*)s->part_ml.p; a.part_acc = (float*)s->part_acc.p;
         const void* o_in = s->att.p;
-        if (!l.latent()) {
+        if (l.recurrent()) {
+            KrSvLin q{};
+            q.kind = d.mixer_kind; q.z = hz; q.ld = l.n_h; q.heads = d.heads; q.dim = d.dim; q.vdim = d.vdim; q.rot_dims = d.rot_dims;
+            q.cs = d.rot_dims ? (const float2*)s->ropes[l.rope_id].cs.p : nullptr;
+            const float isd = (float)(1.0 / std::sqrt((double)d.dim));
+            q.q_scale = d.mixer_kind == KR_SERVE_MIX_MLSTM ? isd : 1.0f; q.k_scale = d.mixer_kind == KR_SERVE_MIX_RETENTION ? isd : 1.0f;
+            q.decay = (const float*)l.decay.p; q.i_bias = (const float*)l.i_bias.p; q.f_bias = (const float*)l.f_bias.p; q.gate_cap = d.gate_cap;
+            q.state = (float*)l.lin_state.p; q.state_stride = l.lin_state_stride; q.nm = (float*)l.lin_nm.p; q.nm_stride = l.lin_nm_stride;
+            q.ent_off = d_eoff; q.ent_slot = d_eslot; q.n_entries = n_entries; q.pos = d_pos; q.T = T;
+            q.o = (float*)s->lin_o.p; q.norm_w = d.lin_norm_weight ? (const float*)l.lin_norm.p : nullptr; q.eps = c.norm_eps; q.out = s->att.p;
+            { Timer tm(s, 3); kr_sv_lin_scan(q, st); }
+            { Timer tm(s, 2); kr_sv_lin_out(q, s->f32, st); }
+        } else if (!l.latent()) {
             a.qkv = hz; a.ldq = l.n_h; a.rot_dims = d.rot_dims; a.rot_interleaved = d.rot_interleaved; a.unit_norm = d.qk_unit_norm; a.own_kv = d.kv_from < 0;
             a.q_norm_w = (const float*)l.q_norm.p; a.k_norm_w = (const float*)l.k_norm.p;
             a.cs = d.rot_dims ? (const float2*)s->ropes[l.rope_id].cs.p : nullptr;
             a.vpool = kvl.vpool.p; a.ldk = d.kv_heads * d.dim; a.ldv = d.kv_heads * d.vdim;
             a.v_mix = d.v_mix; a.v_lambda = (const float*)l.vmix.p; a.v_first = (float*)s->v_first.p;
+            a.q_bias = d.proj_bias ? (const float*)l.q_bias.p : nullptr; a.k_bias = (d.proj_bias && d.kv_from < 0) ? (const float*)l.k_bias.p : nullptr;
+            a.inv_rms = a.inv_rms_out = (float*)s->qk_rms.p; a.v_from_k = d.v_from_k; a.softcap = d.softcap;
+            if (d.out_gate) { a.out_gate = hz + l.off_ogate; a.ld_gate = l.n_h; }
+            if (d.qk_unit_norm == KR_SERVE_QKNORM_WHOLE) { Timer tm(s, 2); kr_sv_qk_rms(a, st); }
             { Timer tm(s, 2); kr_sv_qk_prep(a, s->f32, st); }
             { Timer tm(s, 3); kr_sv_attention(a, s->f32, st); }
         } else {
@@ -668,6 +823,7 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
         if (seq) {
             // the mixer's sublayer ends here; the new x, normed or as it is, is the feed-forward's input (or the next layer's when there is none)
+            res_layer = &l; res_gate_kind = 1; res_to_mixer = !has_ff;
             if (has_ff) residual((const float*)s->mix.p, nullptr, nullptr, nullptr, nullptr, 0, c.post_norm ? &l.post1_w : nullptr, &l.post1_b, true, c.pre_norm ? &l.norm2_w : nullptr, &l.norm2_b);
             else residual((const float*)s->mix.p, nullptr, nullptr, nullptr, nullptr, 0, c.post_norm ? &l.post1_w : nullptr, &l.post1_b, nx != nullptr, (nx && c.pre_norm) ? &nx->norm_w : nullptr,
                           nx ? &nx->norm_b : nullptr);
@@ -686,8 +842,8 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
             int* counts_d = mi; int* seg = mi + E; int* cursor = seg + E + 1; int* src_row = cursor + E; int* row_group = src_row + P; int* pp = row_group + P;
             {
                 Timer tm(s, 4);
-                kr_sv_router_select(hz + l.off_router, l.n_h, s->f32 ? 1 : 2, d.router_bias ? (const float*)l.router_b.p : nullptr, T, E, top, d.groups, d.keep, d.renorm, (int*)s->ids.p,
-                                    (float*)s->wts.p, st);
+                kr_sv_router_select(hz + l.off_router, l.n_h, s->f32 ? 1 : 2, d.router_bias ? (const float*)l.router_b.p : nullptr, d.router_bias, d.router_score, d.group_score, T, E, top,
+                                    d.groups, d.keep, d.renorm, (int*)s->ids.p, (float*)s->wts.p, st);
                 kr_sv_moe_sort((const int*)s->ids.p, T, top, E, counts_d, seg, cursor, src_row, row_group, pp, st);
             }
             g = KrSvGemm{}; g.A = s->h.p; g.lda = W; g.W = l.egu.p; g.w_stride = (size_t)2 * F * W; g.C = (float*)s->gu.p; g.ldc = 2 * F; g.M = P; g.N = 2 * F; g.K = W;
@@ -705,13 +861,14 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
             }
         }
         // x += the layer's sublayers (parallel block) or the feed-forward alone (sequential), and the next layer's input from the same launch
+        res_layer = &l; res_gate_kind = seq ? 2 : 0; res_to_mixer = true;
         if (!seq) residual((const float*)s->mix.p, dense, shared, rows, pair_pos, d.top, nullptr, nullptr, nx != nullptr, (nx && c.pre_norm) ? &nx->norm_w : nullptr, nx ? &nx->norm_b : nullptr);
         else if (has_ff) residual(nullptr, dense, shared, rows, pair_pos, d.top, c.post_norm ? &l.post2_w : nullptr, &l.post2_b, nx != nullptr, (nx && c.pre_norm) ? &nx->norm_w : nullptr,
                                   nx ? &nx->norm_b : nullptr);
         if (s->capture) KR_HIP(hipMemcpyAsync((float*)s->cap.p + (size_t)li * Ts * W, x, Ts * W * 4, hipMemcpyDeviceToDevice, st));
     }
     if (n_want > 0) {
-        { Timer tm(s, 0); kr_sv_norm(x, d_want, (const float*)s->fnorm_w.p, c.norm_bias ? (const float*)s->fnorm_b.p : nullptr, s->hw.p, s->f32, n_want, W, c.norm_eps, c.norm_kind, st); }
+        { Timer tm(s, 0); kr_sv_norm(x, d_want, (const float*)s->fnorm_w.p, c.norm_bias ? (const float*)s->fnorm_b.p : nullptr, s->hw.p, s->f32, n_want, W, c.norm_eps, c.norm_kind, NG, nullptr, st); }
         KrSvGemm g{}; g.A = s->hw.p; g.lda = W; g.W = s->head.p; g.C = (float*)s->logits.p; g.ldc = c.vocab; g.M = n_want; g.N = c.vocab; g.K = W;
         { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
         if (want_amax) { Timer tm(s, 7); kr_sv_argmax((const float*)s->logits.p, n_want, c.vocab, (int*)s->amax.p, st); }
@@ -728,7 +885,7 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         mixin((uint64_t)T); mixin((uint64_t)n_want); mixin(want_amax);
         for (int v : nsplit) mixin((uint64_t)v);
         for (const DevBuf* b : {&s->meta, &s->x, &s->h, &s->qkv, &s->att, &s->mix, &s->gu, &s->y, &s->rows, &s->ffout, &s->ids, &s->wts, &s->rz, &s->moe_i, &s->hw, &s->logits,
-                                &s->amax, &s->part_ml, &s->part_acc, &s->v_first, &s->lq_c, &s->lq_2, &s->lq_n, &s->lq_e, &s->att2, &s->head_i}) mixin((uint64_t)(uintptr_t)b->p);
+                                &s->amax, &s->part_ml, &s->part_acc, &s->v_first, &s->lq_c, &s->lq_2, &s->lq_n, &s->lq_e, &s->att2, &s->head_i, &s->h32, &s->hc, &s->rg, &s->qk_rms, &s->lin_o}) mixin((uint64_t)(uintptr_t)b->p);
         for (const SvRope& r : s->ropes) mixin((uint64_t)(uintptr_t)r.cs.p);
         hipGraphExec_t exec = nullptr;
         for (auto& g : s->graphs) if (g.key == key) exec = g.exec;

@@ -32,9 +32,23 @@ enum { KR_SV_NORM_LAYER = 0, KR_SV_NORM_RMS = 1 };
 enum { KR_SV_ACT_GELU_TANH = 0, KR_SV_ACT_CLAMPED_SWIGLU = 1, KR_SV_ACT_SILU = 2 };
 
 // x[t] = table[tokens[t]]; with h_out also the row in the storage type (the first sublayer's input in a design without input norms)
-void kr_sv_embed(const void* table, bool f32, const int* tokens, float* x, void* h_out, int T, int width, hipStream_t st);
-// out[r] = norm(x[rows ? rows[r] : r]) * w (+ b): two passes over the row, f32; out in the storage type
-void kr_sv_norm(const float* x, const int* rows, const float* w, const float* b, void* out, bool out_f32, int R, int width, float eps, int kind, hipStream_t st);
+// scale: the row is multiplied by it (1 = as it is)
+void kr_sv_embed(const void* table, bool f32, const int* tokens, float* x, void* h_out, int T, int width, float scale, hipStream_t st);
+// out[r] = norm(x[rows ? rows[r] : r]) * w (+ b): two passes over the row, f32; out in the storage type.  groups > 1: the row is normed in that many equal
+// consecutive parts, each by its own statistics.  out32: optional f32 copy of the normed row (the input of a convolution over positions)
+void kr_sv_norm(const float* x, const int* rows, const float* w, const float* b, void* out, bool out_f32, int R, int width, float eps, int kind, int groups, float* out32,
+                hipStream_t st);
+// Input convolution over a request's positions: hc[t] = h[t] + sum_j w[:, j] h(position(t) - taps + 1 + j), channel by channel, zeros before position 0.
+// h of a position comes from this step's rows (h32 [T, width]: the rows of one request stand together, in order) or, for positions before the
+// step's portion, from the request's state: state[slot][position % (taps - 1)][width] f32.  kr_sv_canon_save (any launch after the convolution) keeps
+// the last taps - 1 rows of every portion there.
+struct KrSvCanon {
+    const float* h32; const float* w; int taps;      // w [width, taps]
+    float* state;                                    // [slots][taps - 1][width]
+    const int* slot; const int* pos; int T, width;
+    void* out;                                       // [T, width] storage type
+};
+void kr_sv_canon(const KrSvCanon& c, bool f32, hipStream_t st);
 // cos / sin of pos * inv_freq for every token of the step: cs[t][i] = mult * (cos, sin), the angle formed in double
 void kr_sv_rope_table(const int* pos, const double* inv_freq, float2* cs, int T, int half, float mult, hipStream_t st);
 
@@ -47,6 +61,13 @@ struct KrSvAttn {
     int chunk;                       // > 0: only the keys of the query's own block of `chunk` positions (counted from position 0 of the request)
     const float* slopes;             // [heads] or null: score -= slopes[h] * (query position - key position)
     int v_mix; const float* v_lambda; float* v_first;   // 1: values also kept in v_first [T, kv_heads * vdim]; 2: v <- (1 - *v_lambda) v + *v_lambda v_first
+ // ---- biases, whole-projection norm, values that are the un-normed keys, capped scores, gated output
+    const float* q_bias; const float* k_bias;        // [heads * dim], [kv_heads * dim] or null: added before anything else
+    const float* inv_rms;            // unit_norm == 3: [T, 2] 1 / rms of the whole q and the whole k row (kr_sv_qk_rms), weights q_norm_w [heads * dim], k_norm_w [kv_heads * dim]
+    float* inv_rms_out;              // where kr_sv_qk_rms writes them
+    int v_from_k;                    // the value rows of the cache are the key rows before their norm (no v block in qkv)
+    float softcap;                   // > 0: score <- softcap * tanh(score / softcap) before the distance bias
+    const float* out_gate; int ld_gate;   // [T, ld_gate] f32 or null: head h's output is multiplied by sigmoid(out_gate[t][h])
     const float* sink;               // [heads] or null
     const float2* cs;                // rope table of the step for this layer's rotation
     void* kpool; void* vpool;        // [pages][page_tokens][ldk | ldv] storage type; head g at g * dim | g * vdim of a row (vpool may be kpool: values that are a
@@ -61,15 +82,19 @@ struct KrSvAttn {
 };
 // how many ways to split: fills the chip when the step has few tokens; max_visible = most keys any token of the step sees in this layer
 int kr_sv_attention_splits(int T, int heads, int kv_heads, int dim, int vdim, int ldk, int ldv, bool f32, int max_visible);
-void kr_sv_qk_prep(const KrSvAttn& a, bool f32, hipStream_t st);      // rotation, unit norm, cache append
+void kr_sv_qk_rms(const KrSvAttn& a, hipStream_t st);                 // unit_norm == 3: the two whole-row statistics of every token
+void kr_sv_qk_prep(const KrSvAttn& a, bool f32, hipStream_t st);      // biases, rotation, unit norm, cache append
 void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st);   // windowed softmax with an optional sink over the paged cache
 
 // group-limited top-k router on logits z (rows `ld` floats apart, `parts` column blocks of E that are added): softmax over all experts, the best `keep` of
 // `groups` groups (a group's score = its largest), `top` experts among them; weights = the softmax scores (renorm != 0: divided by their sum).
 // The logits come from kr_sv_gemm: an f32 store multiplies by the f32 gate; a bf16 store by the gate as two bf16 terms (hi + lo rows), which
 // carries 16 bits of the gate's mantissa through the matrix cores.
-// bias [E] or null joins the logits before anything else.
-void kr_sv_router_select(const float* z, int ld, int parts, const float* bias, int T, int E, int top, int groups, int keep, int renorm, int* ids, float* wts, hipStream_t st);
+// bias [E] or null: bias_mode 1 joins the logits before anything else; 2 joins the scores for the choice of groups and experts only (the weights are the
+// scores without it).  score_kind 0: softmax over all experts, 1: sigmoid of every logit.  group_kind 0: a group's score is its largest choice score,
+// 1: the sum of its two largest.  Experts outside the kept groups cannot be chosen, whatever their score.  renorm: weights / (their sum + 1e-20).
+void kr_sv_router_select(const float* z, int ld, int parts, const float* bias, int bias_mode, int score_kind, int group_kind, int T, int E, int top, int groups, int keep,
+                         int renorm, int* ids, float* wts, hipStream_t st);
 // rows of every expert: seg[E + 1], src_row[T * top] (token of sorted row), row_group[T * top], pair_pos[T * top] (sorted row of (token, slot))
 void kr_sv_moe_sort(const int* ids, int T, int top, int E, int* counts, int* seg, int* cursor, int* src_row, int* row_group, int* pair_pos, hipStream_t st);
 // gu rows `ld` floats apart (gate at [0, F), up at [F, 2F)) -> y [M, F] storage type
@@ -82,6 +107,12 @@ struct KrSvResidual {
     const float* post_w; const float* post_b; float mult;
     const float* norm_w; const float* norm_b; void* h_out;
     int T, width, kind; float eps;
+    int groups;                      // > 1: both norms work on that many equal parts of the row
+    float* h32_out;                  // optional f32 copy of the handed-on row
+    const float* gate; int ld_gate; const float* gate_b;   // y <- y * sigmoid(gate[t] + gate_b) element by element, before it joins x (null = no gate)
+    const float* mix_bias;           // [width] or null: added to mix (the output projection's bias)
+    // the input convolution's state: rows of h32_in that are among the last canon_keep of their request's portion go to canon_state[slot][pos % canon_keep]
+    const float* h32_in; float* canon_state; int canon_keep; const int* slot; const int* pos;
 };
 void kr_sv_residual_norm(const KrSvResidual& r, bool out_f32, hipStream_t st);
 
@@ -101,6 +132,32 @@ void kr_sv_latent_prep(const KrSvLatent& a, bool f32, hipStream_t st);
 void kr_sv_latent_q(const KrSvLatent& a, const float* q2, void* qn, float* qe, bool f32, hipStream_t st);
 // rows of a problem grouped by head over [T, heads, *] arrays: seg[h] = h * T, rows[h * T + t] = t * heads + h, group[h * T + t] = h
 void kr_sv_head_rows(int T, int heads, int* seg, int* rows, int* group, hipStream_t st);
+
+// ---- recurrent mixers: per head a matrix state S [dim, vdim] (f32) carried from token to token of a request
+//   retention: S_t = decay_h S_(t-1) + k_t v_t^T,                                   o_t = S_t^T q_t
+//   mlstm:     m_t = max(f_t + m_(t-1), i_t); S_t = exp(f_t + m_(t-1) - m_t) S_(t-1) + exp(i_t - m_t) k_t v_t^T; n_t alike with k_t alone;
+//              o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6);  i = cap(z_i + b_i), f = logsigmoid(cap(z_f + b_f)), cap(z) = gate_cap tanh(z / gate_cap)
+// then o / rms(o) per head (* norm_w) * act(g) -> out in the storage type (act: silu for retention, sigmoid for mlstm).
+// The state of request slot s: S at state + s * state_stride as [heads][vdim][dim]; normaliser and maximum at nm + s * nm_stride as
+// [heads][vdim blocks of 16][dim + 4] (every block of value columns keeps its own copy, so no two workgroups share a word).  A portion that starts at
+// position 0 starts from zeros whatever the slot held.
+struct KrSvLin {
+    int kind;                        // KR_SERVE_MIX_RETENTION (2) | KR_SERVE_MIX_MLSTM (3)
+    float* z; int ld;                // [T, ld] f32: q [heads * dim] | k [heads * dim] | v [heads * vdim] | g [heads * vdim] | (mlstm) z_i [heads] | z_f [heads]
+    int heads, dim, vdim, rot_dims;
+    const float2* cs;                // rotation table of the step [T, rot_dims / 2] (pairs (i, i + rot_dims / 2))
+    float q_scale, k_scale;
+    const float* decay;              // [heads] (retention)
+    const float* i_bias; const float* f_bias; float gate_cap;     // mlstm
+    float* state; size_t state_stride; float* nm; size_t nm_stride;
+    const int* ent_off; const int* ent_slot; int n_entries;       // rows [ent_off[e], ent_off[e + 1]) belong to slot ent_slot[e]
+    const int* pos; int T;
+    float* o;                        // [T, heads * vdim] f32 scratch
+    const float* norm_w; float eps;  // [heads * vdim] or null
+    void* out;                       // [T, heads * vdim] storage type
+};
+void kr_sv_lin_scan(const KrSvLin& a, hipStream_t st);
+void kr_sv_lin_out(const KrSvLin& a, bool f32, hipStream_t st);
 void kr_sv_argmax(const float* logits, int R, int vocab, int* out, hipStream_t st);
 // uniform values in [-amp, amp) from a counter hash of (seed, element); amp = 0 writes zeros
 void kr_sv_fill_uniform(void* p, bool f32, size_t n, uint64_t seed, float amp, hipStream_t st);

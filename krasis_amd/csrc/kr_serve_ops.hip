@@ -46,21 +46,57 @@ __device__ __forceinline__ float sv_block_sum(float v, float* red) {
 }
 
 template <typename T>
-__global__ void __launch_bounds__(256) sv_embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens, float* __restrict__ x, T* __restrict__ h_out, int width) {
+__global__ void __launch_bounds__(256) sv_embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens, float* __restrict__ x, T* __restrict__ h_out, int width,
+                                                       float scale) {
     const int t = blockIdx.x;
     const T* row = table + (size_t)tokens[t] * width;
     for (int c = threadIdx.x; c < width; c += 256) {
-        x[(size_t)t * width + c] = sv_ld(row + c);
-        if (h_out) h_out[(size_t)t * width + c] = row[c];
+        const float v = sv_ld(row + c) * scale;
+        x[(size_t)t * width + c] = v;
+        if (h_out) sv_st(h_out + (size_t)t * width + c, v);
+    }
+}
+
+// statistics of `groups` equal consecutive parts of a row (LDS or global): st[2 g] = mean (0 for an RMS norm), st[2 g + 1] = 1 / sqrt(variance + eps).
+// Wave w of the four takes the parts w, w + 4, ...; the caller makes the row visible before and synchronises after.
+template <int KIND>
+__device__ __forceinline__ void sv_group_stats(const float* xr, int width, int groups, float eps, float* st) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, gw = width / groups;
+    for (int g = wave; g < groups; g += 4) {
+        const float* xg = xr + (size_t)g * gw;
+        float mean = 0.0f;
+        if constexpr (KIND == KR_SV_NORM_LAYER) {
+            float s = 0.0f;
+            for (int c = lane; c < gw; c += 64) s += xg[c];
+            mean = sv_wave_sum(s) / (float)gw;
+        }
+        float q = 0.0f;
+        for (int c = lane; c < gw; c += 64) { const float d = xg[c] - mean; q = __builtin_fmaf(d, d, q); }
+        q = sv_wave_sum(q);
+        if (lane == 0) { st[2 * g] = mean; st[2 * g + 1] = 1.0f / sqrtf(q / (float)gw + eps); }
     }
 }
 
 template <typename T, int KIND>
 __global__ void __launch_bounds__(256) sv_norm_kernel(const float* __restrict__ x, const int* __restrict__ rows, const float* __restrict__ w, const float* __restrict__ b,
-                                                      T* __restrict__ out, int width, float eps) {
+                                                      T* __restrict__ out, int width, float eps, int groups, float* __restrict__ out32) {
     __shared__ float red[4];
+    extern __shared__ float gst[];            // [2 * groups] when the row is normed in parts
     const int r = blockIdx.x;
     const float* xr = x + (size_t)(rows ? rows[r] : r) * width;
+    if (groups > 1) {
+        sv_group_stats<KIND>(xr, width, groups, eps, gst);
+        __syncthreads();
+        const int gw = width / groups;
+        for (int c = threadIdx.x; c < width; c += 256) {
+            const int g = c / gw;
+            float v = (xr[c] - gst[2 * g]) * gst[2 * g + 1] * w[c];
+            if (b) v += b[c];
+            sv_st(out + (size_t)r * width + c, v);
+            if (out32) out32[(size_t)r * width + c] = v;
+        }
+        return;
+    }
     float mean = 0.0f;
     if constexpr (KIND == KR_SV_NORM_LAYER) {
         float s = 0.0f;
@@ -75,7 +111,41 @@ __global__ void __launch_bounds__(256) sv_norm_kernel(const float* __restrict__ 
         float v = (xr[c] - mean) * inv * w[c];
         if (b) v += b[c];
         sv_st(out + (size_t)r * width + c, v);
+        if (out32) out32[(size_t)r * width + c] = v;
     }
+}
+
+// input convolution over positions (KrSvCanon): one thread per (token, channel)
+template <typename T>
+__global__ void __launch_bounds__(256) sv_canon_kernel(const KrSvCanon a, T* __restrict__ out) {
+    const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= a.width) return;
+    const int p = a.pos[t], sl = a.slot[t], K = a.taps - 1;
+    const float* w = a.w + (size_t)c * a.taps;
+    float acc = a.h32[(size_t)t * a.width + c];
+    acc = __builtin_fmaf(w[K], acc, acc);                     // the tap on the token itself
+    for (int d = 1; d <= K; d++) {                            // d positions back
+        const int q = p - d;
+        if (q < 0) break;
+        float hv;
+        if (t - d >= 0 && a.slot[t - d] == sl) hv = a.h32[(size_t)(t - d) * a.width + c];
+        else hv = a.state[((size_t)sl * K + q % K) * a.width + c];
+        acc = __builtin_fmaf(w[K - d], hv, acc);
+    }
+    sv_st(out + (size_t)t * a.width + c, acc);
+}
+
+// unit_norm == 3: 1 / rms over the whole q row (part 0) and the whole k row (part 1) of every token, biases included
+__global__ void __launch_bounds__(256) sv_qk_rms_kernel(const KrSvAttn a) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, part = blockIdx.y;
+    const int n = (part ? a.kv_heads : a.heads) * a.dim;
+    const float* z = a.qkv + (size_t)t * a.ldq + (part ? a.heads * a.dim : 0);
+    const float* b = part ? a.k_bias : a.q_bias;
+    float q = 0.0f;
+    for (int c = threadIdx.x; c < n; c += 256) { const float v = b ? z[c] + b[c] : z[c]; q = __builtin_fmaf(v, v, q); }
+    q = sv_block_sum<4>(q, red);
+    if (threadIdx.x == 0) a.inv_rms_out[(size_t)t * 2 + part] = 1.0f / sqrtf(q / (float)n + a.eps);
 }
 
 __global__ void sv_rope_table_kernel(const int* __restrict__ pos, const double* __restrict__ inv_freq, float2* __restrict__ cs, int T, int half, float mult) {
@@ -100,7 +170,7 @@ __global__ void __launch_bounds__(64) sv_qk_prep_kernel(const KrSvAttn a) {
         const size_t page = (size_t)a.page_table[(size_t)sl * a.table_ld + p / a.page_tokens];
         prow = page * a.page_tokens + (p % a.page_tokens);
     }
-    if (hh >= H + G) {                       // value head: copy, or blend with the values an earlier layer formed for this token
+    if (hh >= H + G) {                       // value head (never launched when the values are the keys): copy, or blend with the values an earlier layer formed for this token
         const int g = hh - H - G;
         const float* v = row + (size_t)H * a.dim + (size_t)G * a.dim + (size_t)g * a.vdim;
         T* dst = (T*)a.vpool + prow * a.ldv + (size_t)g * a.vdim;
@@ -114,9 +184,23 @@ __global__ void __launch_bounds__(64) sv_qk_prep_kernel(const KrSvAttn a) {
         }
         return;
     }
-    float* v = row + (size_t)hh * a.dim;
-    for (int d = lane; d < a.dim; d += 64) hv[d] = v[d];
+ float* v = row + (size_t)hh * a.dim;
+    {
+        const float* bias = hh < H ? a.q_bias : a.k_bias;
+        if (bias) bias += (size_t)(hh < H ? hh : hh - H) * a.dim;
+        for (int d = lane; d < a.dim; d += 64) hv[d] = bias ? v[d] + bias[d] : v[d];
+    }
     __syncthreads();
+    if (a.v_from_k && hh >= H) {             // the value row of this key head: the key as projected
+        T* dst = (T*)a.vpool + prow * a.ldv + (size_t)(hh - H) * a.dim;
+        for (int d = lane; d < a.dim; d += 64) sv_st(dst + d, hv[d]);
+    }
+    if (a.unit_norm == 3) {                  // one statistic for the whole row, a weight per coordinate of the row
+        const float inv3 = a.inv_rms[(size_t)t * 2 + (hh < H ? 0 : 1)];
+        const float* w = hh < H ? a.q_norm_w + (size_t)hh * a.dim : a.k_norm_w + (size_t)(hh - H) * a.dim;
+        for (int d = lane; d < a.dim; d += 64) hv[d] = hv[d] * inv3 * w[d];
+        __syncthreads();
+    }
     if (a.unit_norm == 2) {                  // weighted, before the rotation
         const float* w = hh < H ? a.q_norm_w : a.k_norm_w;
         float s2 = 0.0f;
@@ -279,7 +363,8 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
         SV_STAMP(3);
 #pragma unroll
         for (int r = 0; r < RM; r++) {
-            const float sr = live ? s[r] - slope[r] * (float)(p - j) : -INFINITY;
+            const float sc = a.softcap > 0.0f ? a.softcap * tanhf(s[r] / a.softcap) : s[r];
+            const float sr = live ? sc - slope[r] * (float)(p - j) : -INFINITY;
             const float mn = fmaxf(m[r], sv_wave_max(sr));
             const float alpha = expf(m[r] - mn);               // first block of this wave: exp(-inf) = 0
             const float pj = live ? expf(sr - mn) : 0.0f;
@@ -371,7 +456,10 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
         if (last && a.sink) M = fmaxf(M, a.sink[h0 + r]);
         float L = (last && a.sink) ? expf(a.sink[h0 + r] - M) : 0.0f;
         for (int w = 0; w < 4; w++) { const float mw = ml[(w * RM + r) * 2]; if (mw != -INFINITY) L += ml[(w * RM + r) * 2 + 1] * expf(mw - M); }
-        if (last) sv_st(o + i, accs[i] / L);
+        if (last) {
+            const float gt = a.out_gate ? 1.0f / (1.0f + expf(-a.out_gate[(size_t)t * a.ld_gate + h0 + r])) : 1.0f;
+            sv_st(o + i, accs[i] / L * gt);
+        }
         else {
             const size_t slot = ((size_t)t * a.heads + h0 + r) * a.nsplit + sp;
             a.part_acc[slot * vdim + (i - r * vdim)] = accs[i];
@@ -476,7 +564,8 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
                 for (int i = 0; i < 4; i++) {
                     const int key = j0 + kb * 16 + 4 * qd + i;
                     const bool ok = rv && key <= p_row && key >= lo_row;
-                    st[kb][i] = ok ? st[kb][i] - slope_row * (float)(p_row - key) : -INFINITY;
+                    const float sc = a.softcap > 0.0f ? a.softcap * tanhf(st[kb][i] / a.softcap) : st[kb][i];
+                    st[kb][i] = ok ? sc - slope_row * (float)(p_row - key) : -INFINITY;
                     cm = fmaxf(cm, st[kb][i]);
                 }
             cm = fmaxf(cm, __shfl_xor(cm, 16)); cm = fmaxf(cm, __shfl_xor(cm, 32));
@@ -562,7 +651,10 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
             if (tq < base || tq >= end) continue;
             const int h = g * R + hb * 16 + (r % Rb);
             const float av = accs[acc_at(r, i - r * vdim)];
-            if (last) sv_st((T*)a.out + ((size_t)(t0 + tq) * a.heads + h) * vdim + (i - r * vdim), av * mf[r * 2 + 1]);
+            if (last) {
+                const float gt = a.out_gate ? 1.0f / (1.0f + expf(-a.out_gate[(size_t)(t0 + tq) * a.ld_gate + h])) : 1.0f;
+                sv_st((T*)a.out + ((size_t)(t0 + tq) * a.heads + h) * vdim + (i - r * vdim), av * mf[r * 2 + 1] * gt);
+            }
             else {
                 const size_t slot = ((size_t)(t0 + tq) * a.heads + h) * a.nsplit + sp;
                 a.part_acc[slot * vdim + (i - r * vdim)] = av;
@@ -591,7 +683,7 @@ __global__ void __launch_bounds__(256) sv_attn_merge_kernel(const KrSvAttn a) {
         wsp[a.nsplit] = 1.0f / L;
     }
     __syncthreads();
-    const float inv = wsp[a.nsplit];
+    const float inv = wsp[a.nsplit] * (a.out_gate ? 1.0f / (1.0f + expf(-a.out_gate[(size_t)t * a.ld_gate + h])) : 1.0f);
     T* o = (T*)a.out + ((size_t)t * a.heads + h) * a.vdim;
     for (int d = tid; d < a.vdim; d += 256) {
         float v = 0.0f;
@@ -603,32 +695,37 @@ __global__ void __launch_bounds__(256) sv_attn_merge_kernel(const KrSvAttn a) {
 
 // selection: one wave per token; the scores of the E experts live in LDS
 // z holds the logits as `parts` column blocks of E that are added (a gate stored as two bf16 terms gives two)
-__global__ void __launch_bounds__(64) sv_router_select_kernel(const float* __restrict__ z, int ld, int parts, const float* __restrict__ bias, int E, int top, int groups,
-                                                              int keep, int renorm, int* __restrict__ ids, float* __restrict__ wts) {
-    extern __shared__ float lds[];           // s[E] | gscore[groups] | allowed flags as floats [groups]
-    float* s = lds; float* gs = lds + E; float* gok = gs + groups;
+__global__ void __launch_bounds__(64) sv_router_select_kernel(const float* __restrict__ z, int ld, int parts, const float* __restrict__ bias, int bias_mode, int score_kind,
+                                                              int group_kind, int E, int top, int groups, int keep, int renorm, int* __restrict__ ids, float* __restrict__ wts) {
+    extern __shared__ float lds[];           // s[E] scores | c[E] choice scores | gscore[groups] | allowed flags as floats [groups]
+    float* s = lds; float* cs = lds + E; float* gs = cs + E; float* gok = gs + groups;
     const int t = blockIdx.x, lane = threadIdx.x;
     for (int e = lane; e < E; e += 64) {
         float v = z[(size_t)t * ld + e];
         for (int q = 1; q < parts; q++) v += z[(size_t)t * ld + (size_t)q * E + e];
-        s[e] = bias ? v + bias[e] : v;
+        s[e] = (bias && bias_mode == 1) ? v + bias[e] : v;
     }
     __syncthreads();
-    float mx = -INFINITY;
-    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
-    mx = sv_wave_max(mx);
-    float sum = 0.0f;
-    for (int e = lane; e < E; e += 64) { const float v = expf(s[e] - mx); s[e] = v; sum += v; }
-    __syncthreads();
-    sum = sv_wave_sum(sum);
-    const float inv = 1.0f / sum;
-    for (int e = lane; e < E; e += 64) s[e] *= inv;
+    if (score_kind == 1) {
+        for (int e = lane; e < E; e += 64) s[e] = 1.0f / (1.0f + expf(-s[e]));
+    } else {
+        float mx = -INFINITY;
+        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
+        mx = sv_wave_max(mx);
+        float sum = 0.0f;
+        for (int e = lane; e < E; e += 64) { const float v = expf(s[e] - mx); s[e] = v; sum += v; }
+        __syncthreads();
+        sum = sv_wave_sum(sum);
+        const float inv = 1.0f / sum;
+        for (int e = lane; e < E; e += 64) s[e] *= inv;
+    }
+    for (int e = lane; e < E; e += 64) cs[e] = (bias && bias_mode == 2) ? s[e] + bias[e] : s[e];
     __syncthreads();
     const int per = E / groups;
     for (int gi = lane; gi < groups; gi += 64) {
-        float v = -INFINITY;
-        for (int e = gi * per; e < (gi + 1) * per; e++) v = fmaxf(v, s[e]);
-        gs[gi] = v; gok[gi] = groups == keep ? 1.0f : 0.0f;
+        float v = -INFINITY, v2 = -INFINITY;       // the two largest of the group
+        for (int e = gi * per; e < (gi + 1) * per; e++) { const float c = cs[e]; if (c > v) { v2 = v; v = c; } else if (c > v2) v2 = c; }
+        gs[gi] = (group_kind == 1 && per > 1) ? v + v2 : v; gok[gi] = groups == keep ? 1.0f : 0.0f;
     }
     __syncthreads();
     if (keep < groups) {
@@ -649,8 +746,8 @@ __global__ void __launch_bounds__(64) sv_router_select_kernel(const float* __res
     for (int r = 0; r < top; r++) {
         float bv = -INFINITY; int bi = 0x7fffffff;
         for (int e = lane; e < E; e += 64) {
-            const float v = s[e];
-            if (v >= 0.0f && gok[e / per] != 0.0f && (v > bv || (v == bv && e < bi))) { bv = v; bi = e; }      // a taken expert is marked by a negative score
+            const float v = cs[e];
+            if (v != -INFINITY && gok[e / per] != 0.0f && (v > bv || (v == bv && e < bi))) { bv = v; bi = e; }      // a taken expert is marked by minus infinity
         }
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) {
@@ -658,14 +755,15 @@ __global__ void __launch_bounds__(64) sv_router_select_kernel(const float* __res
             if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
         }
         __syncthreads();
-        if (bi == 0x7fffffff) { bi = 0; bv = 0.0f; }      // fewer allowed experts than `top` (refused on the host): a zero-weight slot
-        else if (lane == 0) s[bi] = -1.0f;
-        if (lane == 0) { ids[(size_t)t * top + r] = bi; wts[(size_t)t * top + r] = bv; }
-        wsum += bv;
+        float wv;
+        if (bi == 0x7fffffff) { bi = 0; wv = 0.0f; }      // fewer allowed experts than `top` (refused on the host): a zero-weight slot
+        else { wv = s[bi]; if (lane == 0) cs[bi] = -INFINITY; }
+        if (lane == 0) { ids[(size_t)t * top + r] = bi; wts[(size_t)t * top + r] = wv; }
+        wsum += wv;
         __syncthreads();
     }
     if (renorm) {
-        const float rinv = 1.0f / wsum;
+        const float rinv = 1.0f / (wsum + 1e-20f);
         for (int r = lane; r < top; r += 64) wts[(size_t)t * top + r] *= rinv;
     }
 }
@@ -731,20 +829,32 @@ __global__ void sv_act_kernel(const float* __restrict__ gu, int ld, T* __restric
     sv_st(y + i, v);
 }
 
-// one workgroup per token: the sublayers' output row is formed in LDS, normed there when the design norms sublayer outputs, added to the residual row,
-// and the new row is written back and handed on in the storage type -- normed for the next sublayer (norm_w) or as it is
+// one workgroup per token: the sublayers' output row is formed in LDS, normed there when the design norms sublayer outputs, gated when the design gates
+// them, added to the residual row, and the new row is written back and handed on in the storage type -- normed for the next sublayer (norm_w) or as it is
 template <typename T, int KIND>
 __global__ void __launch_bounds__(256) sv_residual_norm_kernel(const KrSvResidual a, T* __restrict__ h_out) {
-    extern __shared__ float xr[];            // [width]
+    extern __shared__ float xr[];            // [width] | [2 * groups]
     __shared__ float red[4];
     __shared__ int pp_s[64]; __shared__ float w_s[64];      // the token's expert rows and weights, read once (top <= 64; more fall back to global reads)
     const size_t t = blockIdx.x;
     const int width = a.width, top = a.top;
+    float* gst = xr + width;
     const float* __restrict__ rows = a.rows; const float* __restrict__ mix = a.mix; const float* __restrict__ dense = a.dense; const float* __restrict__ shared = a.shared;
     float* __restrict__ x = a.x;
+    if (a.canon_state) {                     // the mixer's un-convolved input of this token is kept when it is among the last canon_keep of its portion
+        const int K = a.canon_keep, sl = a.slot[t];
+        if ((int)t + K >= a.T || a.slot[t + K] != sl) {
+            float* dst = a.canon_state + ((size_t)sl * K + a.pos[t] % K) * width;
+            for (int c = threadIdx.x; c < width; c += 256) dst[c] = a.h32_in[t * width + c];
+        }
+    }
     const bool staged = rows && top <= 64;
     if (staged && threadIdx.x < top) { pp_s[threadIdx.x] = a.pair_pos[t * top + threadIdx.x]; w_s[threadIdx.x] = a.wts[t * top + threadIdx.x]; }
     if (rows) __syncthreads();
+    auto gate_at = [&](int c) {
+        const float z = a.gate[t * a.ld_gate + c] + (a.gate_b ? a.gate_b[c] : 0.0f);
+        return 1.0f / (1.0f + expf(-z));
+    };
     float s1 = 0.0f;
     for (int c = threadIdx.x; c < width; c += 256) {
         const size_t i = t * width + c;
@@ -761,40 +871,54 @@ __global__ void __launch_bounds__(256) sv_residual_norm_kernel(const KrSvResidua
         if (shared) { ff = any ? ff + shared[i] : shared[i]; any = true; }
         if (dense) { ff = any ? ff + dense[i] : dense[i]; any = true; }
         float d = mix ? mix[i] : 0.0f;
+        if (mix && a.mix_bias) d += a.mix_bias[c];
         if (any) d = mix ? d + ff : ff;
         if (a.post_w) { xr[c] = d; s1 += d; continue; }      // the sum waits for its norm
+        if (a.gate) d *= gate_at(c);
         const float v = x[i] + a.mult * d;
         x[i] = v; xr[c] = v; s1 += v;
     }
     if (a.post_w) {
-        float mean = 0.0f;
-        if constexpr (KIND == KR_SV_NORM_LAYER) mean = sv_block_sum<4>(s1, red) / (float)width;
-        float q = 0.0f;
-        for (int c = threadIdx.x; c < width; c += 256) { const float dv = xr[c] - mean; q = __builtin_fmaf(dv, dv, q); }
-        const float inv = 1.0f / sqrtf(sv_block_sum<4>(q, red) / (float)width + a.eps);
+        float mean = 0.0f, inv = 0.0f;
+        if (a.groups > 1) { __syncthreads(); sv_group_stats<KIND>(xr, width, a.groups, a.eps, gst); __syncthreads(); }
+        else {
+            if constexpr (KIND == KR_SV_NORM_LAYER) mean = sv_block_sum<4>(s1, red) / (float)width;
+            float q = 0.0f;
+            for (int c = threadIdx.x; c < width; c += 256) { const float dv = xr[c] - mean; q = __builtin_fmaf(dv, dv, q); }
+            inv = 1.0f / sqrtf(sv_block_sum<4>(q, red) / (float)width + a.eps);
+        }
+        const int gw = a.groups > 1 ? width / a.groups : width;
         s1 = 0.0f;
         for (int c = threadIdx.x; c < width; c += 256) {
             const size_t i = t * width + c;
+            if (a.groups > 1) { mean = gst[2 * (c / gw)]; inv = gst[2 * (c / gw) + 1]; }
             float y = (xr[c] - mean) * inv * a.post_w[c];
             if (a.post_b) y += a.post_b[c];
+            if (a.gate) y *= gate_at(c);
             const float v = x[i] + a.mult * y;
             x[i] = v; xr[c] = v; s1 += v;
         }
     }
     if (!h_out) return;
     if (!a.norm_w) {
-        for (int c = threadIdx.x; c < width; c += 256) sv_st(h_out + t * width + c, xr[c]);
+        for (int c = threadIdx.x; c < width; c += 256) { sv_st(h_out + t * width + c, xr[c]); if (a.h32_out) a.h32_out[t * width + c] = xr[c]; }
         return;
     }
-    float mean = 0.0f;
-    if constexpr (KIND == KR_SV_NORM_LAYER) mean = sv_block_sum<4>(s1, red) / (float)width;
-    float q = 0.0f;
-    for (int c = threadIdx.x; c < width; c += 256) { const float dv = xr[c] - mean; q = __builtin_fmaf(dv, dv, q); }      // a thread re-reads its own columns
-    const float inv = 1.0f / sqrtf(sv_block_sum<4>(q, red) / (float)width + a.eps);
+    float mean = 0.0f, inv = 0.0f;
+    if (a.groups > 1) { __syncthreads(); sv_group_stats<KIND>(xr, width, a.groups, a.eps, gst); __syncthreads(); }
+    else {
+        if constexpr (KIND == KR_SV_NORM_LAYER) mean = sv_block_sum<4>(s1, red) / (float)width;
+        float q = 0.0f;
+        for (int c = threadIdx.x; c < width; c += 256) { const float dv = xr[c] - mean; q = __builtin_fmaf(dv, dv, q); }      // a thread re-reads its own columns
+        inv = 1.0f / sqrtf(sv_block_sum<4>(q, red) / (float)width + a.eps);
+    }
+    const int gw = a.groups > 1 ? width / a.groups : width;
     for (int c = threadIdx.x; c < width; c += 256) {
+        if (a.groups > 1) { mean = gst[2 * (c / gw)]; inv = gst[2 * (c / gw) + 1]; }
         float v = (xr[c] - mean) * inv * a.norm_w[c];
         if (a.norm_b) v += a.norm_b[c];
         sv_st(h_out + t * width + c, v);
+        if (a.h32_out) a.h32_out[t * width + c] = v;
     }
 }
 
@@ -849,6 +973,125 @@ __global__ void sv_head_rows_kernel(int T, int heads, int* __restrict__ seg, int
     rows[i] = t * heads + h; group[i] = h;
 }
 
+// ---- recurrent mixers (KrSvLin)
+// One WAVE per (request of the step, head, block of 16 value columns): lane = 4 * column + part, and a lane keeps the rows [part * dpr, (part + 1) * dpr) of
+// its column of S in registers for the whole portion (dpr = ceil(dim / 4) <= DP).  The tokens of the portion are walked in order; TB of them at a time are
+// staged in LDS (q and k of the head with the rotation and the scales applied, the 16 value columns, the two gates), so the serial loop reads LDS only.
+// Per token a lane does dpr updates S <- a S + (b v) k and dpr products for o, and the four parts of a column meet through two lane exchanges.
+#define SV_WAVE_SYNC() do { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront"); } while (0)
+template <int KIND, int DP>
+__global__ void __launch_bounds__(64) sv_lin_scan_kernel(const KrSvLin a) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int TB = 8;
+    constexpr bool ML = KIND == 3;
+    const int e = blockIdx.x, h = blockIdx.y, cb = blockIdx.z, lane = threadIdx.x;
+    const int part = lane & 3, cl = lane >> 2, col = cb * 16 + cl;
+    const int dim = a.dim, vdim = a.vdim, H = a.heads, ncb = (vdim + 15) / 16;
+    const int dpr = (dim + 3) / 4, dimp = 4 * dpr;
+    const int t0 = a.ent_off[e], t1 = a.ent_off[e + 1], sl = a.ent_slot[e];
+    const bool fresh = a.pos[t0] == 0, cv = col < vdim;
+    float* Sg = a.state + (size_t)sl * a.state_stride + ((size_t)h * vdim + (cv ? col : 0)) * dim + part * dpr;
+    float* nmg = a.nm + (size_t)sl * a.nm_stride + ((size_t)h * ncb + cb) * (dim + 4);
+    float S[DP], n[DP];
+#pragma unroll
+    for (int r = 0; r < DP; r++) {
+        const int row = part * dpr + r;
+        const bool ok = r < dpr && row < dim && !fresh;
+        S[r] = (ok && cv) ? Sg[r] : 0.0f;
+        n[r] = (ML && ok) ? nmg[row] : 0.0f;
+    }
+    float m = (ML && !fresh) ? nmg[dim] : 0.0f;
+    const float decay = ML ? 0.0f : a.decay[h];
+    float* qs = lds; float* ks = qs + TB * dimp; float* vs = ks + TB * dimp; float* gs = vs + TB * 16;
+    const int half = a.rot_dims / 2;
+    for (int tb = t0; tb < t1; tb += TB) {
+        const int nt = min(TB, t1 - tb);
+        for (int idx = lane; idx < nt * dimp; idx += 64) {
+            const int tt = idx / dimp, d = idx - tt * dimp;
+            const float* zr = a.z + (size_t)(tb + tt) * a.ld + (size_t)h * dim;
+            qs[idx] = d < dim ? zr[d] * a.q_scale : 0.0f;
+            ks[idx] = d < dim ? zr[(size_t)H * dim + d] * a.k_scale : 0.0f;
+        }
+        for (int idx = lane; idx < nt * 16; idx += 64) {
+            const int tt = idx >> 4, c = cb * 16 + (idx & 15);
+            vs[idx] = c < vdim ? a.z[(size_t)(tb + tt) * a.ld + (size_t)2 * H * dim + (size_t)h * vdim + c] : 0.0f;
+        }
+        if (ML && lane < nt) {
+            const float* zg = a.z + (size_t)(tb + lane) * a.ld + (size_t)2 * H * dim + (size_t)2 * H * vdim;
+            float zi = zg[h] + a.i_bias[h], zf = zg[H + h] + a.f_bias[h];
+            if (a.gate_cap > 0.0f) { zi = a.gate_cap * tanhf(zi / a.gate_cap); zf = a.gate_cap * tanhf(zf / a.gate_cap); }
+            gs[2 * lane] = zi;
+            gs[2 * lane + 1] = fminf(zf, 0.0f) - log1pf(expf(-fabsf(zf)));      // log sigmoid
+        }
+        SV_WAVE_SYNC();
+        if (half > 0) {
+            for (int idx = lane; idx < nt * half; idx += 64) {
+                const int tt = idx / half, i = idx - tt * half;
+                const float2 c = a.cs[(size_t)(tb + tt) * half + i];
+                float* qp = qs + tt * dimp; float* kp = ks + tt * dimp;
+                const float qu = qp[i], qv = qp[i + half], ku = kp[i], kv = kp[i + half];
+                qp[i] = qu * c.x - qv * c.y; qp[i + half] = qv * c.x + qu * c.y;
+                kp[i] = ku * c.x - kv * c.y; kp[i + half] = kv * c.x + ku * c.y;
+            }
+            SV_WAVE_SYNC();
+        }
+        for (int tt = 0; tt < nt; tt++) {
+            const float* qp = qs + tt * dimp + part * dpr; const float* kp = ks + tt * dimp + part * dpr;
+            const float v = vs[tt * 16 + cl];
+            float av, bv;
+            if constexpr (ML) {
+                const float ig = gs[2 * tt], fg = gs[2 * tt + 1];
+                const float mn = fmaxf(fg + m, ig);
+                av = expf(fg + m - mn); bv = expf(ig - mn); m = mn;
+            } else { av = decay; bv = 1.0f; }
+            const float bvv = bv * v;
+            float po = 0.0f, pn = 0.0f;
+#pragma unroll
+            for (int r = 0; r < DP; r++) {
+                if (r < dpr) {
+                    const float kr = kp[r], qr = qp[r];
+                    S[r] = __builtin_fmaf(kr, bvv, av * S[r]);
+                    po = __builtin_fmaf(S[r], qr, po);
+                    if constexpr (ML) { n[r] = __builtin_fmaf(bv, kr, av * n[r]); pn = __builtin_fmaf(n[r], qr, pn); }
+                }
+            }
+            po += __shfl_xor(po, 1); po += __shfl_xor(po, 2);
+            if constexpr (ML) {
+                pn += __shfl_xor(pn, 1); pn += __shfl_xor(pn, 2);
+                po = po / (fmaxf(fabsf(pn), expf(-m)) + 1e-6f);
+            }
+            if (part == 0 && cv) a.o[(size_t)(tb + tt) * H * vdim + (size_t)h * vdim + col] = po;
+        }
+        SV_WAVE_SYNC();
+    }
+#pragma unroll
+    for (int r = 0; r < DP; r++) {
+        const int row = part * dpr + r;
+        if (r < dpr && row < dim) {
+            if (cv) Sg[r] = S[r];
+            if (ML && cl == 0) nmg[row] = n[r];
+        }
+    }
+    if (ML && lane == 0) nmg[dim] = m;
+}
+
+// one wave per (token, head): o / rms(o) (* weight) * act(g) -> the output projection's input
+template <typename T>
+__global__ void __launch_bounds__(64) sv_lin_out_kernel(const KrSvLin a, T* __restrict__ out) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, vdim = a.vdim, H = a.heads;
+    const float* o = a.o + ((size_t)t * H + h) * vdim;
+    const float* g = a.z + (size_t)t * a.ld + (size_t)2 * H * a.dim + (size_t)H * vdim + (size_t)h * vdim;
+    float ss = 0.0f;
+    for (int d = lane; d < vdim; d += 64) ss = __builtin_fmaf(o[d], o[d], ss);
+    const float inv = 1.0f / sqrtf(sv_wave_sum(ss) / (float)vdim + a.eps);
+    for (int d = lane; d < vdim; d += 64) {
+        const float gz = g[d], sg = 1.0f / (1.0f + expf(-gz));
+        float v = o[d] * inv;
+        if (a.norm_w) v *= a.norm_w[(size_t)h * vdim + d];
+        sv_st(out + ((size_t)t * H + h) * vdim + d, v * (a.kind == 3 ? sg : gz * sg));
+    }
+}
+
 __global__ void __launch_bounds__(1024) sv_argmax_kernel(const float* __restrict__ logits, int vocab, int* __restrict__ out) {
     __shared__ float bv[16]; __shared__ int bi[16];
     const float* row = logits + (size_t)blockIdx.x * vocab;
@@ -885,15 +1128,17 @@ void kr_sv_fill_uniform(void* p, bool f32, size_t n, uint64_t seed, float amp, h
     else hipLaunchKernelGGL(sv_fill_uniform_kernel<uint16_t>, grid, dim3(256), 0, st, (uint16_t*)p, n, seed, amp);
 }
 
-void kr_sv_embed(const void* table, bool f32, const int* tokens, float* x, void* h_out, int T, int width, hipStream_t st) {
+void kr_sv_embed(const void* table, bool f32, const int* tokens, float* x, void* h_out, int T, int width, float scale, hipStream_t st) {
     if (T <= 0) return;
-    if (f32) hipLaunchKernelGGL(sv_embed_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)table, tokens, x, (float*)h_out, width);
-    else hipLaunchKernelGGL(sv_embed_kernel<uint16_t>, dim3(T), dim3(256), 0, st, (const uint16_t*)table, tokens, x, (uint16_t*)h_out, width);
+    if (f32) hipLaunchKernelGGL(sv_embed_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)table, tokens, x, (float*)h_out, width, scale);
+    else hipLaunchKernelGGL(sv_embed_kernel<uint16_t>, dim3(T), dim3(256), 0, st, (const uint16_t*)table, tokens, x, (uint16_t*)h_out, width, scale);
 }
 
-void kr_sv_norm(const float* x, const int* rows, const float* w, const float* b, void* out, bool out_f32, int R, int width, float eps, int kind, hipStream_t st) {
+void kr_sv_norm(const float* x, const int* rows, const float* w, const float* b, void* out, bool out_f32, int R, int width, float eps, int kind, int groups, float* out32,
+                hipStream_t st) {
     if (R <= 0) return;
-#define SV_NORM(T_, K_) hipLaunchKernelGGL((sv_norm_kernel<T_, K_>), dim3(R), dim3(256), 0, st, x, rows, w, b, (T_*)out, width, eps)
+    const size_t lds = groups > 1 ? (size_t)2 * groups * sizeof(float) : 0;
+#define SV_NORM(T_, K_) hipLaunchKernelGGL((sv_norm_kernel<T_, K_>), dim3(R), dim3(256), lds, st, x, rows, w, b, (T_*)out, width, eps, groups, out32)
     if (kind == KR_SV_NORM_LAYER) { if (out_f32) SV_NORM(float, KR_SV_NORM_LAYER); else SV_NORM(uint16_t, KR_SV_NORM_LAYER); }
     else { if (out_f32) SV_NORM(float, KR_SV_NORM_RMS); else SV_NORM(uint16_t, KR_SV_NORM_RMS); }
 #undef SV_NORM
@@ -905,9 +1150,21 @@ void kr_sv_rope_table(const int* pos, const double* inv_freq, float2* cs, int T,
     hipLaunchKernelGGL(sv_rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, st, pos, inv_freq, cs, T, half, mult);
 }
 
+void kr_sv_qk_rms(const KrSvAttn& a, hipStream_t st) {
+    if (a.T <= 0) return;
+    hipLaunchKernelGGL(sv_qk_rms_kernel, dim3(a.T, 2), dim3(256), 0, st, a);
+}
+
+void kr_sv_canon(const KrSvCanon& c, bool f32, hipStream_t st) {
+    if (c.T <= 0) return;
+    const dim3 grid(c.T, (c.width + 255) / 256);
+    if (f32) hipLaunchKernelGGL(sv_canon_kernel<float>, grid, dim3(256), 0, st, c, (float*)c.out);
+    else hipLaunchKernelGGL(sv_canon_kernel<uint16_t>, grid, dim3(256), 0, st, c, (uint16_t*)c.out);
+}
+
 void kr_sv_qk_prep(const KrSvAttn& a, bool f32, hipStream_t st) {
     if (a.T <= 0) return;
-    const dim3 grid(a.T, a.heads + (a.own_kv ? 2 * a.kv_heads : 0));
+    const dim3 grid(a.T, a.heads + (a.own_kv ? (a.v_from_k ? 1 : 2) * a.kv_heads : 0));
     const size_t lds = (size_t)a.dim * sizeof(float);
     if (f32) hipLaunchKernelGGL(sv_qk_prep_kernel<float>, grid, dim3(64), lds, st, a);
     else hipLaunchKernelGGL(sv_qk_prep_kernel<uint16_t>, grid, dim3(64), lds, st, a);
@@ -1012,10 +1269,11 @@ void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st) {
 #undef SV_ATT
 }
 
-void kr_sv_router_select(const float* z, int ld, int parts, const float* bias, int T, int E, int top, int groups, int keep, int renorm, int* ids, float* wts, hipStream_t st) {
+void kr_sv_router_select(const float* z, int ld, int parts, const float* bias, int bias_mode, int score_kind, int group_kind, int T, int E, int top, int groups, int keep,
+                         int renorm, int* ids, float* wts, hipStream_t st) {
     if (T <= 0) return;
-    const size_t lds = (size_t)(E + 2 * groups) * sizeof(float);
-    hipLaunchKernelGGL(sv_router_select_kernel, dim3(T), dim3(64), lds, st, z, ld, parts, bias, E, top, groups, keep, renorm, ids, wts);
+    const size_t lds = (size_t)(2 * E + 2 * groups) * sizeof(float);
+    hipLaunchKernelGGL(sv_router_select_kernel, dim3(T), dim3(64), lds, st, z, ld, parts, bias, bias_mode, score_kind, group_kind, E, top, groups, keep, renorm, ids, wts);
 }
 
 void kr_sv_moe_sort(const int* ids, int T, int top, int E, int* counts, int* seg, int* cursor, int* src_row, int* row_group, int* pair_pos, hipStream_t st) {
@@ -1041,7 +1299,7 @@ void kr_sv_act(const float* gu, int ld, void* y, bool f32, int M, int F, int kin
 
 void kr_sv_residual_norm(const KrSvResidual& r, bool out_f32, hipStream_t st) {
     if (r.T <= 0) return;
-    const size_t lds = (size_t)r.width * sizeof(float);
+    const size_t lds = (size_t)(r.width + 2 * (r.groups > 1 ? r.groups : 0)) * sizeof(float);
 #define SV_RN(T_, K_) hipLaunchKernelGGL((sv_residual_norm_kernel<T_, K_>), dim3(r.T), dim3(256), lds, st, r, (T_*)r.h_out)
     if (r.kind == KR_SV_NORM_LAYER) { if (out_f32) SV_RN(float, KR_SV_NORM_LAYER); else SV_RN(uint16_t, KR_SV_NORM_LAYER); }
     else { if (out_f32) SV_RN(float, KR_SV_NORM_RMS); else SV_RN(uint16_t, KR_SV_NORM_RMS); }
@@ -1062,6 +1320,23 @@ void kr_sv_head_rows(int T, int heads, int* seg, int* rows, int* group, hipStrea
     const int n = T * heads > heads + 1 ? T * heads : heads + 1;
     if (T <= 0) return;
     hipLaunchKernelGGL(sv_head_rows_kernel, dim3((n + 255) / 256), dim3(256), 0, st, T, heads, seg, rows, group);
+}
+
+void kr_sv_lin_scan(const KrSvLin& a, hipStream_t st) {
+    if (a.T <= 0 || a.n_entries <= 0) return;
+    const int dpr = (a.dim + 3) / 4;
+    const dim3 grid(a.n_entries, a.heads, (a.vdim + 15) / 16);
+    const size_t lds = (size_t)(2 * 8 * 4 * dpr + 8 * 16 + 8 * 2) * sizeof(float);
+#define SV_LIN(K_, DP_) hipLaunchKernelGGL((sv_lin_scan_kernel<K_, DP_>), grid, dim3(64), lds, st, a)
+#define SV_LIN_D(K_) do { if (dpr <= 8) SV_LIN(K_, 8); else if (dpr <= 16) SV_LIN(K_, 16); else if (dpr <= 32) SV_LIN(K_, 32); else SV_LIN(K_, 64); } while (0)
+    if (a.kind == 3) SV_LIN_D(3); else SV_LIN_D(2);
+#undef SV_LIN_D
+#undef SV_LIN
+}
+void kr_sv_lin_out(const KrSvLin& a, bool f32, hipStream_t st) {
+    if (a.T <= 0) return;
+    if (f32) hipLaunchKernelGGL(sv_lin_out_kernel<float>, dim3(a.T, a.heads), dim3(64), 0, st, a, (float*)a.out);
+    else hipLaunchKernelGGL(sv_lin_out_kernel<uint16_t>, dim3(a.T, a.heads), dim3(64), 0, st, a, (uint16_t*)a.out);
 }
 
 void kr_sv_argmax(const float* logits, int R, int vocab, int* out, hipStream_t st) {

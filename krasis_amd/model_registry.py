@@ -81,6 +81,11 @@ class ServeModelSpec:
     post_norm: int = 0
     norm_bias: Optional[int] = None      # None: layer norms carry a bias, RMS norms do not
     residual_mult: float = 1.0
+    norm_groups: int = 0                 # > 1: every norm works on that many equal parts of the row
+    embed_scale: float = 0.0             # 0: the embedding row as it is
+    canon_taps: int = 0                  # > 1: the mixers read h + a causal convolution of h over the request's positions
+    res_gate: int = 0                    # 1: sublayer outputs are gated by sigmoid(W h + b) before they join the stream
+    extra: Optional[dict] = None         # per-layer arrays the design's config carries instead of the checkpoint (tensor name -> float32 array)
 
 
 _ARCHITECTURES: Dict[str, Callable[[dict], ServeModelSpec]] = {}
@@ -233,6 +238,101 @@ def pamulix_spec(cfg: dict) -> ServeModelSpec:
 
 
 register_architecture("Pamulix", pamulix_spec)
+
+
+# ---- Midisun: pre-normed sequential layers x <- x + gate1 * mixer(h1 + conv(h1)), x <- x + gate2 * ff(h2), h = RMS norm in groups, gate = sigmoid(W h + b)
+# element by element, conv = a short causal convolution over the request's positions whose last inputs belong to the request's state.  Three mixers.
+# 'attention': biased q / k / o projections, values = the keys before their norm, one RMS statistic over the whole q (k) row with a full-size weight,
+# capped scores, a distance bias slope_h * (i - j), a sliding window, a learned sink in the denominator, a per-head sigmoid gate on the output.
+# 'retention': rotated q / k (half-split pairs), S <- decay_h S + k v^T with k / sqrt(dim), o = S^T q, per-head unit RMS, times silu(W_g h).
+# 'mlstm': S and a normaliser n under exponential input and sigmoid forget gates kept stable by a running maximum, capped gate pre-activations,
+# per-head unit RMS with a weight, times sigmoid(W_g h).  Feed-forward: SiLU-gated dense, or SiLU-gated experts behind a sigmoid router whose choice
+# (not its weights) is corrected by a bias and limited to the groups with the best top-two sums; weights renormalised over the chosen experts.
+def _midisun_tensors(spec: ServeModelSpec) -> Iterator[Tuple[int, str, int, str]]:
+    yield -1, "embed", 0, "embed"
+    yield -1, "final_norm_w", 0, "final.norm"
+    yield -1, "head", 0, "head"
+    for i, l in enumerate(spec.layers):
+        p = f"l{i}"
+        yield i, "norm_w", 0, f"{p}.norm1"
+        if spec.canon_taps > 1:
+            yield i, "canon", 0, f"{p}.canon1"
+        yield i, "res_gate1", 0, f"{p}.rg1"
+        yield i, "res_gate1_b", 0, f"{p}.rg1.b"
+        yield i, "q", 0, f"{p}.mix.q"
+        yield i, "k", 0, f"{p}.mix.k"
+        yield i, "out_gate", 0, f"{p}.mix.g"
+        yield i, "o", 0, f"{p}.mix.o"
+        if l.mixer_kind == S.MIX_ATTENTION:
+            for r, n in (("q_bias", "q.b"), ("k_bias", "k.b"), ("o_bias", "o.b"), ("q_norm", "q.norm"), ("k_norm", "k.norm"), ("sink", "sink")):
+                yield i, r, 0, f"{p}.mix.{n}"
+        else:
+            yield i, "v", 0, f"{p}.mix.v"
+            if l.mixer_kind == S.MIX_MLSTM:
+                for r, n in (("lin_norm", "norm"), ("igate", "i"), ("igate_b", "i.b"), ("fgate", "f"), ("fgate_b", "f.b")):
+                    yield i, r, 0, f"{p}.mix.{n}"
+            else:
+                yield i, "lin_decay", 0, f"{p}.mix.decay"      # from config.json (spec.extra), not from the checkpoint
+        if l.mlp_kind != S.MLP_NONE:
+            yield i, "norm2_w", 0, f"{p}.norm2"
+            yield i, "res_gate2", 0, f"{p}.rg2"
+            yield i, "res_gate2_b", 0, f"{p}.rg2.b"
+        if l.mlp_kind == S.MLP_DENSE:
+            for r in ("gate", "up", "down"):
+                yield i, r, 0, f"{p}.mlp.{r}"
+        elif l.mlp_kind == S.MLP_MOE:
+            yield i, "router", 0, f"{p}.mlp.router"
+            yield i, "router_bias", 0, f"{p}.mlp.correction"
+            for e in range(l.experts):
+                for r in ("gate", "up", "down"):
+                    yield i, f"expert_{r}", e, f"{p}.mlp.e{e}.{r}"
+
+
+def midisun_spec(cfg: dict) -> ServeModelSpec:
+    layers: List[S.LayerSpec] = []
+    extra: Dict[str, np.ndarray] = {}
+    for i, lc in enumerate(cfg["layers"]):
+        kind, m = lc.get("type"), lc["mixer"]
+        if kind == "attention":
+            l = S.LayerSpec(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
+                            qk_unit_norm=S.QKNORM_WHOLE, scale=float(m["scale"]), window=int(m["mask"]["size"]), has_sink=S.SINK_TENSOR, dist_bias=1, dist_bias_exp=8.0,
+                            proj_bias=1, v_from_k=1, softcap=float(m["softcap"]), out_gate=S.OGATE_HEAD_SIGMOID)
+            if l.vdim != l.dim:
+                raise ValueError(f"layer {i}: the values are the keys, so vdim {l.vdim} must equal dim {l.dim}")
+        elif kind == "retention":
+            rot = m.get("rot") or {}
+            l = S.LayerSpec(heads=int(m["heads"]), kv_heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]), mixer_kind=S.MIX_RETENTION,
+                            rot_dims=int(rot.get("dims", 0)), rot_interleaved=0, rot_base=float(rot.get("base", 10000.0)))
+            dec = np.asarray(m["decay"], np.float32)
+            if dec.shape != (l.heads,):
+                raise ValueError(f"layer {i}: {dec.size} decays for {l.heads} heads")
+            extra[f"l{i}.mix.decay"] = dec
+        elif kind == "mlstm":
+            l = S.LayerSpec(heads=int(m["heads"]), kv_heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]), mixer_kind=S.MIX_MLSTM,
+                            gate_cap=float(m["gate_cap"]), lin_norm_weight=1)
+        else:
+            raise ValueError(f"layer {i}: mixer type {kind!r} is not part of this design")
+        mlp = lc.get("mlp")
+        if mlp is not None:
+            if mlp.get("kind") == "dense":
+                l.mlp_kind, l.ff, l.dense_act = S.MLP_DENSE, int(mlp["ff"]), S.ACT_SILU
+            elif mlp.get("kind") == "moe":
+                r, ex = mlp["router"], mlp["expert"]
+                g = r.get("groups") or {}
+                l.mlp_kind, l.experts, l.top = S.MLP_MOE, int(r["experts"]), int(r["top"])
+                l.groups, l.keep = int(g.get("count", 1)), int(g.get("keep", g.get("count", 1)))
+                l.renorm, l.router_bias, l.router_score, l.group_score = 1, S.RBIAS_CHOICE, S.RSCORE_SIGMOID, S.GSCORE_TOP2
+                l.expert_ff, l.expert_act = int(ex["ff"]), S.ACT_SILU
+            else:
+                raise ValueError(f"layer {i}: feed-forward kind {mlp.get('kind')!r}")
+        layers.append(l)
+    return ServeModelSpec(vocab=int(cfg["vocab"]), width=int(cfg["width"]), norm_kind=S.NORM_RMS, norm_eps=float(cfg["norm"]["eps"]), layers=layers,
+                          tensors=_midisun_tensors, block_kind=S.BLOCK_SEQUENTIAL, pre_norm=1, post_norm=0, norm_bias=0,
+                          norm_groups=int(cfg["norm"].get("groups", 1)), embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)),
+                          canon_taps=int((cfg.get("canon") or {}).get("taps", 0)), res_gate=1, extra=extra)
+
+
+register_architecture("Midisun", midisun_spec)
 
 
 def read_config(model_dir: str) -> dict:

@@ -24,7 +24,8 @@ class BatchEngine:
         self.spec = spec
         self.store = S.ServeStore(spec.vocab, spec.width, spec.layers, dtype=_DTYPES[dtype], norm_kind=spec.norm_kind, norm_eps=spec.norm_eps,
                                   max_slots=max_slots, pool_tokens=max_tokens, device=device, build=build, block_kind=spec.block_kind, pre_norm=spec.pre_norm,
-                                  post_norm=spec.post_norm, norm_bias=spec.norm_bias, residual_mult=spec.residual_mult)
+                                  post_norm=spec.post_norm, norm_bias=spec.norm_bias, residual_mult=spec.residual_mult, norm_groups=spec.norm_groups,
+                                  embed_scale=spec.embed_scale, canon_taps=spec.canon_taps, res_gate=spec.res_gate)
         self.vocab = spec.vocab
         self._slot: Dict[object, int] = {}
 
@@ -32,14 +33,16 @@ class BatchEngine:
     def load_safetensors(self, path: str) -> None:
         from .model_registry import SafetensorsFile
         f = SafetensorsFile(path)
+        extra = getattr(self.spec, "extra", None) or {}
         for layer, role, index, name in self.spec.tensors(self.spec):
-            self.store.set_tensor(layer, role, f.get(name), index)
+            self.store.set_tensor(layer, role, extra[name] if name in extra else f.get(name), index)
         self.store.finalize()
 
     def load_arrays(self, arrays: Dict[str, np.ndarray]) -> None:
         """tensors by checkpoint name: float32, or uint16 bf16 bit patterns"""
+        extra = getattr(self.spec, "extra", None) or {}
         for layer, role, index, name in self.spec.tensors(self.spec):
-            self.store.set_tensor(layer, role, arrays[name], index)
+            self.store.set_tensor(layer, role, extra[name] if name in extra else arrays[name], index)
         self.store.finalize()
 
     def load_synthetic(self, seed: int = 1, amp: float = 1.0) -> None:

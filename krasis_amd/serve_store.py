@@ -17,8 +17,12 @@ NORM_LAYER, NORM_RMS = 0, 1
 MLP_NONE, MLP_DENSE, MLP_MOE = 0, 1, 2
 ACT_GELU_TANH, ACT_CLAMPED_SWIGLU, ACT_SILU = 0, 1, 2
 BLOCK_PARALLEL, BLOCK_SEQUENTIAL = 0, 1
-MIX_ATTENTION, MIX_LATENT = 0, 1
-QKNORM_NONE, QKNORM_AFTER_ROT, QKNORM_WEIGHTED = 0, 1, 2
+MIX_ATTENTION, MIX_LATENT, MIX_RETENTION, MIX_MLSTM = 0, 1, 2, 3
+QKNORM_NONE, QKNORM_AFTER_ROT, QKNORM_WEIGHTED, QKNORM_WHOLE = 0, 1, 2, 3
+RBIAS_NONE, RBIAS_LOGIT, RBIAS_CHOICE = 0, 1, 2
+RSCORE_SOFTMAX, RSCORE_SIGMOID = 0, 1
+GSCORE_MAX, GSCORE_TOP2 = 0, 1
+OGATE_NONE, OGATE_HEAD_SIGMOID = 0, 1
 SINK_NONE, SINK_TENSOR, SINK_ZERO = 0, 1, 2
 ROT_LINEAR, ROT_BY_PARTS = 0, 1
 VMIX_NONE, VMIX_FIRST, VMIX_BLEND = 0, 1, 2
@@ -26,12 +30,14 @@ PAGE_TOKENS = 64
 ROLES = {n: i for i, n in enumerate(["embed", "final_norm_w", "final_norm_b", "head", "norm_w", "norm_b", "q", "k", "v", "o", "sink", "gate", "up", "down",
                                      "router", "expert_gate", "expert_up", "expert_down", "shared_gate", "shared_up", "shared_down",
                                      "norm2_w", "norm2_b", "post1_w", "post1_b", "post2_w", "post2_b", "q_norm", "k_norm", "vmix", "router_bias",
-                                     "dq", "dq_norm", "uq", "dkv", "dkv_norm", "uk", "uv"])}
+                                     "dq", "dq_norm", "uq", "dkv", "dkv_norm", "uk", "uv",
+                                     "q_bias", "k_bias", "o_bias", "out_gate", "canon", "res_gate1", "res_gate1_b", "res_gate2", "res_gate2_b",
+                                     "lin_norm", "lin_decay", "igate", "igate_b", "fgate", "fgate_b"])}
 
 
 @dataclass
 class LayerSpec:
-    """One layer: a mixer (attention, or attention through latents) and a feed-forward, beside or after one another (field meanings: `kr_serve_layer`
+    """One layer: a mixer (attention, attention through latents, or a recurrent matrix state) and a feed-forward, beside or after one another (field meanings: `kr_serve_layer`
     in include/krasis_hip.h)."""
     heads: int
     kv_heads: int
@@ -72,12 +78,21 @@ class LayerSpec:
     dist_bias_exp: float = 8.0
     v_mix: int = VMIX_NONE
     router_bias: int = 0
+    proj_bias: int = 0
+    v_from_k: int = 0
+    softcap: float = 0.0
+    out_gate: int = OGATE_NONE
+    gate_cap: float = 0.0
+    lin_norm_weight: int = 0
+    router_score: int = RSCORE_SOFTMAX
+    group_score: int = GSCORE_MAX
 
 
 class ServeStore:
     def __init__(self, vocab: int, width: int, layers: Sequence[LayerSpec], dtype: int = BF16, norm_kind: int = NORM_LAYER, norm_eps: float = 1e-5,
                  max_slots: int = 4, pool_tokens: int = 4096, page_tokens: int = PAGE_TOKENS, device: int = 0, build: bool = False,
-                 block_kind: int = BLOCK_PARALLEL, pre_norm: int = 1, post_norm: int = 0, norm_bias: Optional[int] = None, residual_mult: float = 1.0):
+                 block_kind: int = BLOCK_PARALLEL, pre_norm: int = 1, post_norm: int = 0, norm_bias: Optional[int] = None, residual_mult: float = 1.0,
+                 norm_groups: int = 0, embed_scale: float = 0.0, canon_taps: int = 0, res_gate: int = 0):
         self._lib = load_serve_library(build=build)
         self.vocab, self.width, self.layers, self.dtype = vocab, width, list(layers), dtype
         self.page_tokens = page_tokens
@@ -86,7 +101,7 @@ class ServeStore:
         if norm_bias is None:
             norm_bias = int(norm_kind == NORM_LAYER)
         cfg = ServeConfigC(vocab, width, len(self.layers), dtype, norm_kind, norm_eps, max_slots, page_tokens, pool_tokens, block_kind, pre_norm, post_norm, norm_bias,
-                           residual_mult)
+                           residual_mult, norm_groups, embed_scale, canon_taps, res_gate)
         arr = (ServeLayerC * len(self.layers))()
         for i, l in enumerate(self.layers):
             for f in fields(LayerSpec):
