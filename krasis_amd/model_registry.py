@@ -291,6 +291,7 @@ def _midisun_tensors(spec: ServeModelSpec) -> Iterator[Tuple[int, str, int, str]
 def midisun_spec(cfg: dict) -> ServeModelSpec:
     layers: List[S.LayerSpec] = []
     extra: Dict[str, np.ndarray] = {}
+    taps = int((cfg.get("canon") or {}).get("taps", 0))      # one tap or none: the mixers read their normed input as it is
     for i, lc in enumerate(cfg["layers"]):
         kind, m = lc.get("type"), lc["mixer"]
         if kind == "attention":
@@ -329,7 +330,7 @@ def midisun_spec(cfg: dict) -> ServeModelSpec:
     return ServeModelSpec(vocab=int(cfg["vocab"]), width=int(cfg["width"]), norm_kind=S.NORM_RMS, norm_eps=float(cfg["norm"]["eps"]), layers=layers,
                           tensors=_midisun_tensors, block_kind=S.BLOCK_SEQUENTIAL, pre_norm=1, post_norm=0, norm_bias=0,
                           norm_groups=int(cfg["norm"].get("groups", 1)), embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)),
-                          canon_taps=int((cfg.get("canon") or {}).get("taps", 0)), res_gate=1, extra=extra)
+                          canon_taps=taps if taps > 1 else 0, res_gate=1, extra=extra)
 
 
 register_architecture("Midisun", midisun_spec)

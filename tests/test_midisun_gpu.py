@@ -1,0 +1,545 @@
+"""The batched serving store (kr_serve_*) with the Midisun design against the plain float64 restatement in tests/oracle_midisun.py.
+
+Small random models of several shapes; every comparison is between what the store's step function returns (logits, or the residual stream after each
+layer) and the oracle run on the whole sequence.  The f32 store is held to 2e-4 of the stream's scale; the bf16 store is judged row by row, since a
+router's close call may fall the other way for single tokens."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from tests import oracle_midisun as O
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def engine(cfg, W, dtype="float32", max_tokens=1024, max_slots=4):
+    from krasis_amd import model_registry as R
+    from krasis_amd.scheduler import BatchEngine
+    eng = BatchEngine(R.midisun_spec(cfg), dtype=dtype, max_tokens=max_tokens, max_slots=max_slots)
+    eng.load_arrays(W)
+    return eng
+
+
+def rel(got, ref):
+    """largest row error, relative to the root mean square of the reference rows"""
+    d = np.asarray(got, np.float64) - ref
+    return float(np.sqrt((d ** 2).mean(-1)).max() / np.sqrt((ref ** 2).mean()))
+
+
+def tokens(cfg, n, seed):
+    return [int(t) for t in np.random.default_rng(seed).integers(0, cfg["vocab"], n)]
+
+
+# sizes differ from layer to layer; key / value heads fewer than query heads; value width unlike key width in the recurrent layers; rotation on a part
+# of a head; routers with top == experts, top == 1, three groups of which two are kept, one group; a layer without feed-forward; three norm groups
+def cfg_varied():
+    return O.make_config(width=96, vocab=101, groups=3, taps=3, embed_scale=1.7, layers=[
+        O.layer(O.mlstm(3, 20, 12, gate_cap=6.0), O.moe(12, 3, 24, groups=3, keep=2)),
+        O.layer(O.attn(6, 3, 16, 11, scale=0.31, softcap=5.0), O.dense(40)),
+        O.layer(O.retention(4, 24, 16, [0.9, 0.97, 0.99, 0.999], rot_dims=12, base=300.0), None),
+        O.layer(O.attn(4, 4, 24, 70, scale=0.2, softcap=11.0), O.moe(8, 8, 16)),
+        O.layer(O.mlstm(2, 8, 40, gate_cap=15.0), O.moe(5, 1, 12)),
+        O.layer(O.retention(5, 12, 20, [0.5, 0.8, 0.95, 0.98, 0.995], base=50.0), O.moe(6, 2, 12, groups=2, keep=1)),
+    ])
+
+
+def cfg_wide():
+    """rows that are multiples of 16 bytes and head shapes of the matrix-instruction attention (four and sixteen heads per key head); recurrent heads of
+    64 and 128 keys; five taps; a window longer than two pages"""
+    return O.make_config(width=128, vocab=260, eps=1e-6, groups=8, taps=5, embed_scale=0.8, layers=[
+        O.layer(O.attn(8, 2, 64, 150, scale=0.12, softcap=25.0), O.moe(16, 4, 32, groups=4, keep=2)),
+        O.layer(O.retention(2, 64, 32, [0.98, 0.9995], base=1e4), O.dense(96)),
+        O.layer(O.mlstm(2, 128, 48, gate_cap=9.0), O.moe(4, 2, 48)),
+        O.layer(O.attn(16, 1, 32, 70, scale=0.2, softcap=40.0), None),
+        O.layer(O.retention(4, 32, 64, [0.9, 0.99, 0.999, 1.0], rot_dims=16, base=777.0), O.moe(6, 2, 24, groups=3, keep=1)),
+    ])
+
+
+@pytest.mark.parametrize("make,n", [(cfg_varied, 75), (cfg_wide, 200)])
+def test_every_layer_and_logits_f32(make, n):
+    cfg = make(); W = O.random_weights(cfg, 1); toks = tokens(cfg, n, 2)
+    ref_logits, ref_streams = O.forward(cfg, W, toks)
+    eng = engine(cfg, W)
+    eng.store.set_capture(True)
+    logits, amax = eng.step([("a", toks, list(range(n)))])
+    streams = eng.store.read_capture(n)
+    for li in range(len(cfg["layers"])):
+        assert rel(streams[li], ref_streams[li]) < 2e-4, f"layer {li}"
+    assert rel(logits, ref_logits) < 2e-4
+    assert np.array_equal(amax, logits.argmax(-1))
+
+
+@pytest.mark.parametrize("make,n", [(cfg_varied, 75), (cfg_wide, 150)])
+def test_bf16_store_close_to_oracle(make, n):
+    cfg = make(); W = {k: O.bf16_round(v) for k, v in O.random_weights(cfg, 3).items()}; toks = tokens(cfg, n, 4)
+    ref_logits, _ = O.forward(cfg, W, toks)
+    eng = engine(cfg, W, "bfloat16")
+    logits, _ = eng.step([("a", toks, list(range(n)))])
+    # a token whose candidate experts score within the bf16 rounding of the router's input may take another one: the rows are judged one by one
+    d = logits - ref_logits
+    e = np.sqrt((d ** 2).mean(-1)) / np.sqrt((ref_logits ** 2).mean())
+    assert np.median(e) < 3e-2 and (e < 6e-2).mean() >= 0.85
+
+
+def small_model(layers, width=64, vocab=50, **kw):
+    return O.make_config(width=width, vocab=vocab, layers=layers, **kw)
+
+
+def quiet_input_gate(W):
+    """input gates far below zero: the running maximum stays near its start value 0 and exp(-m) decides the denominator of the first tokens"""
+    W["l0.mix.i.b"] = np.full_like(W["l0.mix.i.b"], -7.0)
+
+
+def loud_sinks(W):
+    W["l0.mix.sink"] = np.full_like(W["l0.mix.sink"], 6.0)
+
+
+def negative_choice_scores(W):
+    """corrections below -1: every choice score is negative, and experts outside the kept groups must still lose against them"""
+    W["l0.mlp.correction"] = (W["l0.mlp.correction"] - 2.0).astype(np.float32)
+
+
+MECHANISMS = [
+    ("attention_window_1_sees_itself_only", [O.layer(O.attn(2, 1, 8, 1, scale=0.6), None)], {}, None),
+    ("attention_window_3", [O.layer(O.attn(4, 4, 16, 3, scale=0.6), None)], {}, None),
+    ("attention_window_64_is_a_page", [O.layer(O.attn(2, 1, 8, 64, scale=0.6), None)], {}, None),
+    ("attention_cap_bites", [O.layer(O.attn(4, 2, 16, 30, scale=2.0, softcap=1.5), None)], {}, None),
+    ("attention_loud_sinks", [O.layer(O.attn(4, 2, 16, 30, scale=0.4), None)], {}, loud_sinks),
+    ("attention_on_the_matrix_path", [O.layer(O.attn(4, 4, 32, 9, scale=0.4), None)], {}, None),
+    ("attention_thirty_two_heads_on_one_key_head", [O.layer(O.attn(32, 1, 32, 11, scale=0.4), None)], {}, None),
+    ("retention_full_rotation", [O.layer(O.retention(2, 16, 16, [0.9, 0.99]), None)], {}, None),
+    ("retention_partial_rotation_odd_sizes", [O.layer(O.retention(3, 20, 7, [0.7, 0.95, 1.0], rot_dims=6, base=40.0), None)], {}, None),
+    ("retention_wide_values", [O.layer(O.retention(1, 8, 72, [0.93], base=100.0), None)], {}, None),
+    ("retention_keys_of_200", [O.layer(O.retention(2, 200, 24, [0.96, 0.999], rot_dims=64), None)], {}, None),
+    ("mlstm_plain", [O.layer(O.mlstm(2, 16, 16), None)], {}, None),
+    ("mlstm_quiet_input_gate", [O.layer(O.mlstm(3, 12, 20, gate_cap=8.0), None)], {}, quiet_input_gate),
+    ("mlstm_tight_cap_odd_sizes", [O.layer(O.mlstm(5, 10, 9, gate_cap=0.7), None)], {}, None),
+    ("no_convolution", [O.layer(O.attn(2, 2, 8, 5), O.dense(24))], {"taps": 1}, None),
+    ("two_taps_one_norm_group_no_embedding_scale", [O.layer(O.mlstm(2, 8, 8), O.dense(24))], {"taps": 2, "groups": 1, "embed_scale": 1.0}, None),
+    ("seven_taps_sixteen_norm_groups", [O.layer(O.retention(2, 8, 8, [0.9, 0.8]), O.dense(24))], {"taps": 7, "groups": 16}, None),
+    ("experts_top_3_of_10_in_5_groups_keep_2", [O.layer(O.attn(2, 1, 8, 20), O.moe(10, 3, 12, groups=5, keep=2))], {}, None),
+    ("experts_negative_choice_scores", [O.layer(O.attn(2, 1, 8, 20), O.moe(9, 2, 12, groups=3, keep=1))], {}, negative_choice_scores),
+    ("experts_all_chosen", [O.layer(O.mlstm(2, 8, 8), O.moe(4, 4, 12))], {}, None),
+    ("experts_top_1_groups_of_one", [O.layer(O.retention(2, 8, 8, [0.9, 0.8]), O.moe(6, 1, 12, groups=6, keep=2))], {}, None),
+]
+
+
+@pytest.mark.parametrize("name,layers,kw,patch", MECHANISMS, ids=[m[0] for m in MECHANISMS])
+def test_each_mechanism_alone(name, layers, kw, patch):
+    cfg = small_model(layers, **kw)
+    W = O.random_weights(cfg, 5)
+    if patch:
+        patch(W)
+    toks = tokens(cfg, 40, 6)
+    ref_logits, ref_streams = O.forward(cfg, W, toks)
+    eng = engine(cfg, W)
+    eng.store.set_capture(True)
+    logits, _ = eng.step([("a", toks, list(range(40)))])
+    got = eng.store.read_capture(40)
+    for li in range(len(layers)):
+        assert rel(got[li], ref_streams[li]) < 2e-4, (name, li)
+    assert rel(logits, ref_logits) < 2e-4, name
+    # and the same tokens one by one, through the cache and the state
+    rows = [eng.step([("d", [t], [0])])[0][0] for t in toks]
+    assert rel(np.stack(rows), ref_logits) < 2e-4, name
+
+
+def test_the_oracle_feels_every_mechanism(monkeypatch):
+    """the oracle itself: leaving out the sink, the cap, the distance bias, the whole-row norm, the convolution, the residual gate, the correction, the
+    group limit, the rotation or the start value of the running maximum moves its result far beyond the tolerance the store is held to"""
+    cfg = small_model([O.layer(O.attn(4, 2, 16, 12, scale=1.0, softcap=2.0), O.moe(9, 2, 12, groups=3, keep=1)),
+                       O.layer(O.retention(2, 16, 12, [0.9, 0.99], rot_dims=8, base=30.0), O.dense(24)), O.layer(O.mlstm(2, 8, 12, gate_cap=4.0), None)])
+    W = O.random_weights(cfg, 5); W["l2.mix.i.b"] = np.full_like(W["l2.mix.i.b"], -3.0); toks = tokens(cfg, 30, 6)
+    base, _ = O.forward(cfg, W, toks)
+
+    def changed(**patch):
+        with monkeypatch.context() as m:
+            for k, v in patch.items():
+                m.setattr(O, k, v)
+            return O.forward(cfg, W, toks)[0]
+
+    def weights(**patch):
+        W2 = dict(W); W2.update(patch)
+        return O.forward(cfg, W2, toks)[0]
+    assert rel(changed(head_slopes=lambda H: np.zeros(H)), base) > 1e-2
+    assert rel(changed(tanh_cap=lambda z, cap: z), base) > 1e-2
+    assert rel(changed(input_convolution=lambda h, w: h), base) > 2e-2
+    assert rel(changed(rotate_half_pairs=lambda v, pos, dims, b: v), base) > 1e-2
+    assert rel(changed(grouped_norm=lambda x, w, g, eps: O.unit_rms(x, eps) * w), base) > 1e-2
+    assert rel(weights(**{"l0.mix.sink": np.full(4, -30.0, np.float32)}), base) > 1e-2
+    assert rel(weights(**{"l0.mlp.correction": np.zeros(9, np.float32)}), base) > 1e-2
+    assert rel(weights(**{"l0.rg1.b": np.full(64, 30.0, np.float32)}), base) > 1e-2
+    cfg2 = json.loads(json.dumps(cfg)); cfg2["layers"][0]["mlp"]["router"]["groups"] = {"count": 1, "keep": 1}
+    assert rel(O.forward(cfg2, W, toks)[0], base) > 1e-2
+    # the running maximum starts at 0: started at the first input gate instead, the first tokens' denominators differ
+    q = np.ones((3, 1, 4)); k = np.ones((3, 1, 4)) * 0.1; v = np.ones((3, 1, 2))
+    o = O.mlstm_recurrence(q, k, v, np.full((3, 1), -5.0), np.full((3, 1), -0.1))
+    assert abs(o[0, 0, 0] - np.exp(-4.9) * 0.4 / (np.exp(0.1) + 1e-6)) < 1e-9      # m_1 = max(-0.1 + 0, -5) = -0.1
+
+
+# ---------------------------------------------------------------------------------------------------------------- one key that decides
+def peaked_attention_model(window, dim=32, width=64, vocab=40):
+    """attention that finds ONE key: no convolution and no biases in this layer, so that a token's key and query depend on the token alone; the query
+    projection is steered so that the query of token 1 points along the key of token 0.  After the whole-row norms that key scores about 1.2 * dim
+    against O(sqrt(dim)) for any other: whether token 0 is inside the query's window decides the output at a token 1.  Two heads: slopes 1 / 16 and
+    1 / 256, so the second head still prefers the key hundreds of positions back."""
+    cfg = small_model([O.layer(O.attn(2, 1, dim, window, scale=1.2, softcap=60.0), None)], width=width, vocab=vocab, groups=4)
+    W = O.random_weights(cfg, 11)
+    W["l0.canon1"][:] = 0.0
+    for n in ("l0.mix.q.b", "l0.mix.k.b"):
+        W[n][:] = 0.0
+    W["l0.mix.q.norm"][:] = 1.0; W["l0.mix.k.norm"][:] = 1.0
+    x = W["embed"].astype(np.float64) * cfg["embedding"]["scale"]
+    h = O.grouped_norm(x[:2], W["l0.norm1"].astype(np.float64), 4, cfg["norm"]["eps"])
+    k0 = W["l0.mix.k"].astype(np.float64) @ h[0]
+    steer = np.outer(np.concatenate([k0, k0]), h[1]) / (h[1] @ h[1])
+    W["l0.mix.q"] = (0.3 * W["l0.mix.q"] + 2.0 * steer).astype(np.float32)
+    return cfg, W
+
+
+def needle_sequence(vocab, n, needle_at, query_at, seed):
+    """random tokens 2.., token 0 (the needle) once, token 1 (the query) once"""
+    t = [int(x) for x in np.random.default_rng(seed).integers(2, vocab, n)]
+    t[needle_at] = 0; t[query_at] = 1
+    return t
+
+
+def whole_then_decoded(eng, toks, ref, qpos, n):
+    want = [qpos - 1, qpos, qpos + 1]
+    whole, _ = eng.step([("w", toks, want)])
+    assert rel(whole, ref[want]) < 2e-4
+    eng.finish("w")
+    cut = qpos - 2          # the same positions decoded one token at a time after a prompt that ends before the query
+    eng.step([("d", toks[:cut], [])])
+    got = []
+    for p in range(cut, n):
+        lg, _ = eng.step([("d", [toks[p]], [0])])
+        got.append(lg[0])
+    assert rel(np.stack(got), ref[cut:]) < 2e-4
+
+
+@pytest.mark.parametrize("window,qpos", [(7, 40), (40, 119), (64, 191), (65, 129), (130, 300), (300, 640)])
+@pytest.mark.parametrize("inside", [True, False])
+def test_key_on_the_windows_last_position_and_one_beyond_prompt_and_decode(window, qpos, inside):
+    cfg, W = peaked_attention_model(window)
+    n = qpos + 3
+    needle = qpos - (window - 1) if inside else qpos - window
+    toks = needle_sequence(cfg["vocab"], n, needle, qpos, 13)
+    ref, _ = O.forward(cfg, W, toks)
+    # the oracle's own sensitivity: the needle on the other side of the edge changes the query's logits by hundreds of times the tolerance
+    ref2, _ = O.forward(cfg, W, needle_sequence(cfg["vocab"], n, qpos - window if inside else qpos - (window - 1), qpos, 13))
+    assert rel(ref2[qpos:qpos + 1], ref[qpos:qpos + 1]) > 0.05
+    whole_then_decoded(engine(cfg, W, max_tokens=1408), toks, ref, qpos, n)
+
+
+@pytest.mark.parametrize("needle,query", [(63, 64), (63, 127), (64, 128), (0, 1), (0, 63), (127, 128), (1, 128)])
+def test_keys_at_page_borders(needle, query):
+    cfg, W = peaked_attention_model(128)
+    n = 140
+    toks = needle_sequence(cfg["vocab"], n, needle, query, 19)
+    ref, _ = O.forward(cfg, W, toks)
+    eng = engine(cfg, W)
+    cut = (query // 64) * 64 if query % 64 else query - 1       # the prompt cut exactly at the page border before the query, then decoded
+    cut = max(cut, 1)
+    eng.step([("a", toks[:cut], [])])
+    got = []
+    for p in range(cut, query + 1):
+        lg, _ = eng.step([("a", [toks[p]], [0])])
+        got.append(lg[0])
+    assert rel(np.stack(got), ref[cut:query + 1]) < 2e-4
+
+
+def remembering_model(kind, width=64, vocab=12, fillers=range(2, 8)):
+    """a recurrent layer that keeps a token for hundreds of positions: decays / forget gates next to one, no rotation on most of every head, no
+    convolution (keys and queries depend on the token alone), and the query of token 1 set to the part of token 0's key that is orthogonal to the keys
+    of all filler tokens: at the query, the hundreds of fillers in the state count for nothing and token 0 for everything"""
+    if kind == "retention":
+        mixer = O.retention(2, 32, 24, [0.9995, 0.9999], rot_dims=8, base=1e6)
+    else:
+        mixer = O.mlstm(2, 32, 24, gate_cap=12.0)
+    cfg = small_model([O.layer(mixer, None)], width=width, vocab=vocab, groups=4)
+    W = O.random_weights(cfg, 12)
+    W["l0.canon1"][:] = 0.0
+    W["l0.mix.o"] *= 4.0
+    if kind == "mlstm":
+        W["l0.mix.f.b"][:] = 9.0; W["l0.mix.f"] *= 0.1
+        W["l0.mix.i"] *= 0.1; W["l0.mix.i.b"][:] = 0.0
+    x = W["embed"].astype(np.float64) * cfg["embedding"]["scale"]
+    h = O.grouped_norm(x, W["l0.norm1"].astype(np.float64), 4, cfg["norm"]["eps"])
+    keys = (h @ W["l0.mix.k"].astype(np.float64).T).reshape(vocab, 2, 32)
+    keys[:, :, :8] = 0.0                                       # the rotated pairs (i, i + 4), i < 4, stay out of the match
+    target = np.zeros((2, 32))
+    for hd in range(2):
+        F = keys[list(fillers), hd]                            # [fillers, 32]
+        k0 = keys[0, hd]
+        target[hd] = k0 - F.T @ np.linalg.lstsq(F.T, k0, rcond=None)[0]
+    q = 0.2 * W["l0.mix.q"].astype(np.float64)
+    q += np.outer(4.0 * target.reshape(-1) - q @ h[1], h[1]) / (h[1] @ h[1])      # token 1's query is exactly 4 x target
+    W["l0.mix.q"] = q.astype(np.float32)
+    return cfg, W
+
+
+@pytest.mark.parametrize("kind", ["retention", "mlstm"])
+def test_far_token_among_hundreds_through_the_state(kind):
+    """the one matching key was fed 700 positions earlier, in another step; the state carried it"""
+    cfg, W = remembering_model(kind)
+    n = 760
+    toks = needle_sequence(8, n, 40, 740, 17)                    # fillers 2 .. 7
+    ref, _ = O.forward(cfg, W, toks)
+    toks_moved = list(toks); toks_moved[40] = 5
+    ref_moved, _ = O.forward(cfg, W, toks_moved)
+    assert rel(ref_moved[740:741], ref[740:741]) > 0.1           # the far token carries the answer
+    eng = engine(cfg, W, max_tokens=832)
+    eng.step([("a", toks[:300], []), ("other", toks_moved[:90], [])])
+    eng.step([("a", toks[300:700], [])])
+    lg, _ = eng.step([("a", toks[700:], [40]), ("other", toks_moved[90:95], [])])
+    assert rel(lg, ref[740:741]) < 2e-4
+    eng.finish("a")
+    eng.step([("b", toks[:739], [])])
+    eng.step([("b", toks[739:740], [])])
+    lg, _ = eng.step([("b", toks[740:741], [0])])
+    assert rel(lg, ref[740:741]) < 2e-4
+
+
+def test_first_tokens_of_a_sequence():
+    cfg = cfg_varied(); W = O.random_weights(cfg, 21); toks = tokens(cfg, 6, 22)
+    ref, _ = O.forward(cfg, W, toks)
+    eng = engine(cfg, W)
+    one, _ = eng.step([("one", toks[:1], [0])])
+    assert rel(one, ref[:1]) < 2e-4
+    two, _ = eng.step([("two", toks[:2], [0, 1])])
+    assert rel(two, ref[:2]) < 2e-4
+    nxt, _ = eng.step([("one", toks[1:2], [0])])
+    assert rel(nxt, ref[1:2]) < 2e-4
+    rest, _ = eng.step([("one", toks[2:4], [0, 1]), ("two", toks[2:3], [0])])       # the convolution reaches back over three separate steps
+    assert rel(rest, np.stack([ref[2], ref[3], ref[2]])) < 2e-4
+    last, _ = eng.step([("two", toks[3:6], [0, 1, 2])])
+    assert rel(last, ref[3:6]) < 2e-4
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-4), ("bfloat16", 4e-2)])
+def test_prefill_equals_token_by_token_decode(dtype, tol):
+    cfg = cfg_varied(); W = {k: O.bf16_round(v) for k, v in O.random_weights(cfg, 23).items()}; n = 90; toks = tokens(cfg, n, 24)
+    ref, _ = O.forward(cfg, W, toks)
+    eng = engine(cfg, W, dtype)
+    whole, _ = eng.step([("w", toks, list(range(n)))])
+    rows = []
+    for p in range(n):
+        lg, _ = eng.step([("d", [toks[p]], [0])])
+        rows.append(lg[0])
+    dec = np.stack(rows)
+    if dtype == "float32":
+        assert rel(whole, ref) < tol and rel(dec, ref) < tol
+    else:       # bf16: a close call of the router may fall the other way for a few tokens
+        for got in (whole, dec):
+            e = np.sqrt(((got - ref) ** 2).mean(-1)) / np.sqrt((ref ** 2).mean())
+            assert np.median(e) < 3e-2 and (e < tol + 2e-2).mean() >= 0.85
+
+
+@pytest.mark.parametrize("sizes", [[2] * 30, [3, 2, 7, 2, 64, 5, 65, 2, 31, 2, 9], [37, 3, 3, 37, 37, 5, 11, 25, 24, 2], [1, 128, 2, 60], [1, 1, 2, 1, 3, 1, 1, 4]])
+def test_portions_of_several_sizes(sizes):
+    cfg = cfg_wide(); W = O.random_weights(cfg, 25); n = sum(sizes); toks = tokens(cfg, n, 26)
+    ref, _ = O.forward(cfg, W, toks)
+    eng = engine(cfg, W)
+    at, rows = 0, []
+    for s in sizes:
+        lg, _ = eng.step([("c", toks[at:at + s], list(range(s)))])
+        rows.append(lg); at += s
+    assert rel(np.concatenate(rows), ref) < 2e-4
+
+
+@pytest.mark.parametrize("make", [cfg_varied, cfg_wide])
+def test_unequal_requests_in_one_batch_equal_each_alone(make):
+    cfg = make(); W = O.random_weights(cfg, 27)
+    lens = {"a": 70, "b": 9, "c": 131, "d": 33}
+    toks = {k: tokens(cfg, n, 30 + i) for i, (k, n) in enumerate(lens.items())}
+    refs = {k: O.forward(cfg, W, t)[0] for k, t in toks.items()}
+    eng = engine(cfg, W, max_tokens=512)
+    # a schedule that mixes portions with single tokens: every request advances by its own stride; 0 = the request sits this step out
+    stride = {"a": [17, 1, 0, 30, 1, 20], "b": [2, 1, 1, 0, 0, 4], "c": [64, 1, 65, 0, 1], "d": [1, 1, 31]}
+    at = {k: 0 for k in lens}
+    got = {k: [] for k in lens}
+    step = 0
+    while any(at[k] < lens[k] for k in lens):
+        entries, owners = [], []
+        for k in lens:
+            if at[k] >= lens[k]:
+                continue
+            s = stride[k][step] if step < len(stride[k]) else 1
+            s = min(s, lens[k] - at[k])
+            if s == 0:
+                continue
+            entries.append((k, toks[k][at[k]:at[k] + s], list(range(s)))); owners.append((k, s)); at[k] += s
+        lg, _ = eng.step(entries)
+        o = 0
+        for k, s in owners:
+            got[k].append(lg[o:o + s]); o += s
+        step += 1
+    for k in lens:
+        assert rel(np.concatenate(got[k]), refs[k]) < 2e-4, k
+
+
+def test_pages_and_slots_are_used_again():
+    """a pool of five pages and four slots: requests come and go; the later ones run in pages and slots -- cache rows, convolution rows, matrix states --
+    that the earlier ones gave back"""
+    cfg = cfg_varied(); W = O.random_weights(cfg, 31)
+    eng = engine(cfg, W, max_tokens=320, max_slots=4)
+    assert eng.store.free_pages() == 5
+    seqs = [tokens(cfg, n, 40 + i) for i, n in enumerate([130, 60, 64, 100, 65, 190, 20, 129])]
+    refs = [O.forward(cfg, W, t)[0] for t in seqs]
+    a, _ = eng.step([(0, seqs[0], [129]), (1, seqs[1], [59]), (2, seqs[2], [63])])      # 3 + 1 + 1 pages: the pool is full
+    assert eng.store.free_pages() == 0
+    with pytest.raises(RuntimeError):
+        eng.step([(3, seqs[3], [0])])                        # no page left: refused, nothing changed
+    assert rel(a, np.stack([refs[0][129], refs[1][59], refs[2][63]])) < 2e-4
+    eng.finish(0); eng.finish(3)                            # request 3 was admitted (slot) but holds no page
+    assert eng.store.free_pages() == 3
+    b, _ = eng.step([(3, seqs[3], [99]), (4, seqs[4][:40], [39])])          # 2 + 1 pages, out of request 0's
+    assert rel(b, np.stack([refs[3][99], refs[4][39]])) < 2e-4
+    eng.finish(1); eng.finish(2)
+    c, _ = eng.step([(4, seqs[4][40:], [24]), (3, [seqs[3][0]], [])])      # request 4 crosses into a second page (one that request 1 or 2 held)
+    assert rel(c, refs[4][64:65]) < 2e-4
+    eng.finish(3); eng.finish(4)
+    assert eng.store.free_pages() == 5
+    d, _ = eng.step([(5, seqs[5], [0, 189]), (6, seqs[6], [19])])
+    assert rel(d, np.stack([refs[5][0], refs[5][189], refs[6][19]])) < 2e-4
+    eng.finish(5)
+    e, _ = eng.step([(7, seqs[7][:1], [0])])                # one token into a slot whose state another request filled
+    f, _ = eng.step([(7, seqs[7][1:], [127]), (6, [3], [0])])
+    assert rel(np.concatenate([e, f[:1]]), np.stack([refs[7][0], refs[7][128]])) < 2e-4
+
+
+def test_long_decoding_through_pages_and_windows():
+    cfg = cfg_wide(); W = O.random_weights(cfg, 33); n = 330; toks = tokens(cfg, n, 34)
+    ref, _ = O.forward(cfg, W, toks)
+    eng = engine(cfg, W)
+    eng.step([("a", toks[:20], [])])
+    rows = []
+    for p in range(20, n):
+        lg, _ = eng.step([("a", [toks[p]], [0])])
+        rows.append(lg[0])
+    assert rel(np.stack(rows), ref[20:]) < 2e-4
+
+
+def greedy_oracle(cfg, W, prompt, n_new):
+    seq, out, margins = list(prompt), [], []
+    for _ in range(n_new):
+        lg = O.forward(cfg, W, seq)[0][-1]
+        top = np.sort(lg)[-2:]
+        margins.append(float(top[1] - top[0]))
+        out.append(int(lg.argmax())); seq.append(out[-1])
+    return out, min(margins)
+
+
+def test_greedy_generation_through_the_scheduler():
+    """five prompts, four slots, a pool that cannot hold all at once, a step budget that cuts prompts into portions"""
+    cfg = cfg_varied(); W = O.random_weights(cfg, 35)
+    prompts = [tokens(cfg, n, 50 + i) for i, n in enumerate([45, 3, 70, 18, 29])]
+    eng = engine(cfg, W, max_tokens=256, max_slots=4)
+    outs = eng.generate(prompts, 6, token_budget=32)
+    assert eng.store.free_pages() == 4 and not eng.live()
+    for p, o in zip(prompts, outs):
+        want, margin = greedy_oracle(cfg, W, p, 6)
+        if margin > 1e-3:                                   # a near-tie of the two best logits may fall either way in f32
+            assert o == want
+        else:
+            assert o[0] == want[0] or margin < 1e-3
+
+
+def test_sampling_uses_the_frameworks_sampler():
+    cfg = cfg_varied(); W = O.random_weights(cfg, 37); p = tokens(cfg, 12, 38)
+    eng = engine(cfg, W)
+    a = eng.generate([p], 8, temperature=0.8, top_k=5, top_p=0.9, seed=7)
+    b = eng.generate([p], 8, temperature=0.8, top_k=5, top_p=0.9, seed=7)
+    assert a == b and len(a[0]) == 8
+    g = eng.generate([p], 8)
+    k1 = eng.generate([p], 8, temperature=1.3, top_k=1, seed=3)      # top_k = 1 is greedy whatever the temperature
+    assert g == k1
+
+
+def test_checkpoint_directory_command_line_and_trace_replay(tmp_path):
+    cfg = cfg_varied(); W = {k: O.bf16_round(v) for k, v in O.random_weights(cfg, 39).items()}
+    model = str(tmp_path / "model"); O.write_checkpoint(model, cfg, W)
+    from krasis_amd import model_registry as R
+    assert R.model_family(R.read_config(model)) == "serve:Midisun"
+    p1, p2 = tokens(cfg, 20, 60), tokens(cfg, 7, 61)
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    out = subprocess.run([sys.executable, "-m", "krasis_amd", "generate", "--model", model, "--dtype", "float32", "--max-new-tokens", "4",
+                          "--prompt", ",".join(map(str, p1)), "--prompt", ",".join(map(str, p2))], env=env, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    lines = [json.loads(x) for x in out.stdout.splitlines() if x.startswith("{")]
+    for p, line in zip((p1, p2), lines):
+        want, margin = greedy_oracle(cfg, W, p, 4)
+        assert line["prompt"] == p and (line["tokens"] == want or margin < 1e-3)
+    # trace replay: two requests, portions beside single tokens, one ends early and its slot is used again
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": p1[:11], "want": [10]}, {"id": "y", "tokens": p2[:2], "want": []}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": p1[11:12], "want": [0]}, {"id": "y", "tokens": p2[2:], "want": [0, 4]}], "end": ["y"]},
+             {"step": 2, "entries": [{"id": "x", "tokens": p1[12:], "want": []}], "end": []},
+             {"step": 3, "entries": [{"id": "z", "tokens": p2, "want": [6]}], "end": ["x", "z"]}]
+    outdir = str(tmp_path / "out")
+    r = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", model, "--dtype", "float32", "--out", outdir, "--max-tokens", "128"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [x for x in r.stdout.splitlines() if x.startswith("done")] == ["done 0", "done 1", "done 2", "done 3"]
+    r1, r2 = O.forward(cfg, W, p1)[0], O.forward(cfg, W, p2)[0]
+    V = cfg["vocab"]
+    g0 = np.fromfile(os.path.join(outdir, "0.f32"), "<f4").reshape(-1, V)
+    g1 = np.fromfile(os.path.join(outdir, "1.f32"), "<f4").reshape(-1, V)
+    g3 = np.fromfile(os.path.join(outdir, "3.f32"), "<f4").reshape(-1, V)
+    assert not os.path.exists(os.path.join(outdir, "2.f32"))
+    assert rel(g0, r1[10:11]) < 2e-4 and rel(g1, np.stack([r1[11], r2[2], r2[6]])) < 2e-4 and rel(g3, r2[6:7]) < 2e-4
+
+
+def test_store_refuses_what_it_cannot_run():
+    from krasis_amd import serve_store as S
+    seq = dict(block_kind=S.BLOCK_SEQUENTIAL, norm_kind=S.NORM_RMS)
+    with pytest.raises(ValueError):          # a convolution in a block whose sublayers share one input
+        S.ServeStore(50, 32, [S.LayerSpec(heads=4, kv_heads=2, dim=8, vdim=8)], canon_taps=3)
+    with pytest.raises(ValueError):          # norm groups that do not divide the width
+        S.ServeStore(50, 32, [S.LayerSpec(heads=4, kv_heads=2, dim=8, vdim=8)], norm_groups=5, **seq)
+    with pytest.raises(ValueError):          # values that are the keys, of another width
+        S.ServeStore(50, 32, [S.LayerSpec(heads=4, kv_heads=2, dim=8, vdim=12, v_from_k=1)], **seq)
+    with pytest.raises(ValueError):          # a window on a recurrent mixer
+        S.ServeStore(50, 32, [S.LayerSpec(heads=4, kv_heads=4, dim=8, vdim=8, mixer_kind=S.MIX_RETENTION, window=5)], **seq)
+    with pytest.raises(ValueError):          # grouped key / value heads on a recurrent mixer
+        S.ServeStore(50, 32, [S.LayerSpec(heads=4, kv_heads=2, dim=8, vdim=8, mixer_kind=S.MIX_MLSTM)], **seq)
+    st = S.ServeStore(50, 32, [S.LayerSpec(heads=4, kv_heads=4, dim=8, vdim=6, mixer_kind=S.MIX_RETENTION, rot_dims=4, rot_interleaved=0)], res_gate=1, **seq)
+    with pytest.raises(RuntimeError):
+        st.finalize()                                         # tensors missing
+    with pytest.raises(ValueError):
+        st.set_tensor(0, "sink", np.zeros(4, np.float32))     # a recurrent mixer has no sink
+    with pytest.raises(ValueError):
+        st.set_tensor(0, "lin_decay", np.zeros(3, np.float32))  # wrong shape
+    with pytest.raises(ValueError):
+        st.set_tensor(0, "igate", np.zeros((4, 32), np.float32))  # gates belong to the other recurrent mixer
+
+
+def test_graph_replays_equal_eager_steps():
+    """decode steps replay a captured graph from their second visit on; every replay is compared with a store that runs eagerly, with eager steps of
+    other shapes (a prompt portion of a third request) and host synchronisation between the replays"""
+    cfg = cfg_wide(); W = O.random_weights(cfg, 41)
+    a, b = tokens(cfg, 150, 42), tokens(cfg, 150, 43)
+    c = tokens(cfg, 60, 44)
+    eng_g, eng_e = engine(cfg, W, "bfloat16"), engine(cfg, W, "bfloat16")
+    eng_e.store.set_use_graph(False)
+    for eng in (eng_g, eng_e):
+        eng.step([("a", a[:30], []), ("b", b[:7], [])])
+    for i in range(100):
+        entries = [("a", [a[30 + i]], [0]), ("b", [b[7 + i]], [0])]
+        lg, am = eng_g.step(entries)
+        le, ae = eng_e.step(entries)
+        assert np.array_equal(lg, le) and np.array_equal(am, ae), i
+        if i % 25 == 10:                                    # an eager step of another shape in between
+            part = c[(i // 25) * 15:(i // 25) * 15 + 15]
+            lg, _ = eng_g.step([("c", part, [14])]); le, _ = eng_e.step([("c", part, [14])])
+            assert np.array_equal(lg, le)
+    assert eng_g.store.graph_replays() >= 60 and eng_e.store.graph_replays() == 0
+    lg, _ = eng_g.step([("a", [a[130]], [0])])
+    ref = O.forward(cfg, {k: O.bf16_round(v) for k, v in W.items()}, a[:131])[0]
+    e = np.sqrt(((lg[0] - ref[130]) ** 2).mean()) / np.sqrt((ref ** 2).mean())
+    assert e < 5e-2
