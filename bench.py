@@ -347,9 +347,9 @@ def parse():
                          "sizes -- prompt pass and decode throughput, kernel-family times -- beside the closest model of the decode graph (GQA + softmax top-k MoE, INT4) at "
                          "the same sizes; prints its own JSON line")
     ap.add_argument("--arch-sizes", default="small,large", help="sizes of --arch-compare (ARCH_SIZES)")
-    ap.add_argument("--arch-design", default="lomutar", choices=["lomutar", "pamulix"],
-                    help="which layer-described design --arch-compare measures: lomutar (beside the decode graph's GQA + MoE model) or pamulix (beside Lomutar, "
-                         "both on the batched serving store, at the same layer sizes)")
+    ap.add_argument("--arch-design", default="lomutar", choices=["lomutar", "pamulix", "midisun"],
+                    help="which layer-described design --arch-compare measures: lomutar (beside the decode graph's GQA + MoE model), pamulix or midisun (beside "
+                         "Lomutar, both on the batched serving store, at the same layer sizes)")
     return ap.parse_args()
 
 
@@ -579,6 +579,92 @@ def arch_compare_pamulix(args):
         r["prefill"]["attention_frac_of_f32_matrix_peak"] = r["prefill"]["attention_family_TFLOPs"] / F32_MATRIX_PEAK_TFLOPS
         for B, d in m["decode"].items():
             byts = 2.0 * (L * (w_att + (min(E, B * k) + 1) * 3 * W * F + E * W * 2) + V * W)
+            r["decode_b%d" % B] = {"tok_s": B / d["s_per_step"], "ms_per_step": d["s_per_step"] * 1e3, "weight_bytes_per_step": byts,
+                                   "frac_of_hbm_peak": byts / d["s_per_step"] / 1e9 / HBM_PEAK_GBS, "family_ms": {n: round(v, 4) for n, v in zip(SERVE_FAMILIES, d["family_ms"])},
+                                   "gemm_family_frac_of_hbm_peak": byts / (d["family_ms"][1] * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        res["lomutar"] = r
+        del eng; gc.collect()
+        out["sizes"][name] = res
+    flush_native_stdout()
+    print(json.dumps(out), flush=True)
+    return out
+
+
+def midisun_serve_engine(z, kinds):
+    """A Midisun model with random bf16 weights on the batched serving store at the layer sizes z (ARCH_SIZES); kinds: one letter per layer, A = windowed
+    attention (values = keys, capped scores, distance bias, sink, head gates), R = retention, M = mLSTM; recurrent heads have the size's head count and
+    head size for keys and values.  Every layer: grouped RMS norms, a four-tap input convolution, gated residuals, a sigmoid router over the size's
+    experts in four groups of which two are kept."""
+    from krasis_amd import model_registry as R, scheduler as SCH, serve_store as S
+    W, H, G, D, E, k, F, V, P = (z[c] for c in ("width", "heads", "kv_heads", "dim", "experts", "top", "ff", "vocab", "prompt"))
+    moe = dict(mlp_kind=S.MLP_MOE, experts=E, top=k, groups=4, keep=2, renorm=1, router_bias=S.RBIAS_CHOICE, router_score=S.RSCORE_SIGMOID, group_score=S.GSCORE_TOP2,
+               expert_ff=F, expert_act=S.ACT_SILU)
+    mk = {"A": lambda: S.LayerSpec(heads=H, kv_heads=G, dim=D, vdim=D, qk_unit_norm=S.QKNORM_WHOLE, scale=D ** -0.5, window=z["window"], has_sink=S.SINK_TENSOR, dist_bias=1,
+                                   proj_bias=1, v_from_k=1, softcap=30.0, out_gate=S.OGATE_HEAD_SIGMOID, **moe),
+          "R": lambda: S.LayerSpec(heads=H, kv_heads=H, dim=D, vdim=D, mixer_kind=S.MIX_RETENTION, rot_dims=D, rot_interleaved=0, rot_base=1e6, **moe),
+          "M": lambda: S.LayerSpec(heads=H, kv_heads=H, dim=D, vdim=D, mixer_kind=S.MIX_MLSTM, gate_cap=12.0, lin_norm_weight=1, **moe)}
+    spec = R.ServeModelSpec(V, W, S.NORM_RMS, 1e-5, [mk[c]() for c in kinds], None, block_kind=S.BLOCK_SEQUENTIAL, pre_norm=1, post_norm=0, norm_bias=0, norm_groups=4,
+                            embed_scale=2.0, canon_taps=4, res_gate=1)
+    eng = SCH.BatchEngine(spec, dtype="bfloat16", max_tokens=4 * (P + 256), max_slots=4)
+    eng.load_synthetic(seed=7, amp=1.0)
+    return eng
+
+
+def arch_compare_midisun(args):
+    """The Midisun design beside Lomutar, both on the batched serving store with random bf16 weights, at the layer sizes of ARCH_SIZES.  Four Midisun
+    models per size: the mixed order attention, retention, mLSTM, attention, ... (the throughput), and one mixer kind alone each (what its kernels reach).
+    The recurrent kernels are priced against the f32 vector rate (their products are f32 by the design): 4 (retention) or 6 (mLSTM) flops per state
+    element and token."""
+    import numpy as np
+    from krasis_amd import model_registry as R, scheduler as SCH, serve_store as S
+    out = {"metric": "arch_compare_midisun_vs_lomutar", "unit": "tok/s", "sizes": {}}
+    for name in [x for x in args.arch_sizes.split(",") if x]:
+        z = ARCH_SIZES[name]; W, H, G, D, E, k, F, L, V, P = (z[c] for c in ("width", "heads", "kv_heads", "dim", "experts", "top", "ff", "layers", "vocab", "prompt"))
+        res = {"shape": dict(z)}
+        w_moe_tok = k * 3 * W * F
+        w_gates = 2 * W * W                                       # the two residual gates of a layer
+        w_att = (H * D + G * D + H) * W + W * H * D
+        w_rec = 4 * H * D * W + W * H * D                        # q, k, v, g and the output projection (+ 2 H gate rows for mLSTM)
+        att_flops = 2.0 * 2 * H * D * sum(min(i + 1, z["window"]) for i in range(P))
+        rec_flops = {"R": 4.0 * P * H * D * D, "M": 6.0 * P * H * D * D}
+        order = "".join("ARMA"[i % 4] for i in range(L))
+        for label, kinds in (("mixed_" + order, order), ("attention_only", "A" * L), ("retention_only", "R" * L), ("mlstm_only", "M" * L)):
+            eng = midisun_serve_engine(z, kinds)
+            m = serve_measure(eng, V, P, np.random.default_rng(3), decode_batches=(1, 4) if label.startswith("mixed") else (1,))
+            nA, nR, nM = kinds.count("A"), kinds.count("R"), kinds.count("M")
+            macs_tok = nA * w_att + (nR + nM) * w_rec + nM * 2 * H * W + L * (w_moe_tok + E * W + w_gates)
+            fam = m["prefill_family_ms"]
+            mix_flops = nA * att_flops + nR * rec_flops["R"] + nM * rec_flops["M"]
+            r = {"prefill": {"tok_s": P / m["prefill_s"], "ms": m["prefill_s"] * 1e3, "tokens": P, "family_ms": {n: round(v, 3) for n, v in zip(SERVE_FAMILIES, fam)},
+                             "gemm_family_frac_of_bf16_peak": 2.0 * P * (macs_tok + V * W / P) / (fam[1] * 1e-3) / 1e12 / F16_PEAK_TFLOPS,
+                             "mixer_family_TFLOPs": mix_flops / (fam[3] * 1e-3) / 1e12}}
+            r["prefill"]["mixer_frac_of_f32_peak"] = r["prefill"]["mixer_family_TFLOPs"] / F32_MATRIX_PEAK_TFLOPS
+            for B, d in m["decode"].items():
+                state = 2.0 * 4 * B * (nR + nM) * H * D * D          # the matrix states, read and written, f32
+                byts = 2.0 * (nA * w_att + (nR + nM) * w_rec + L * (min(E, B * k) * 3 * W * F + E * W + w_gates) + V * W) + state
+                r["decode_b%d" % B] = {"tok_s": B / d["s_per_step"], "ms_per_step": d["s_per_step"] * 1e3, "weight_and_state_bytes_per_step": byts,
+                                       "frac_of_hbm_peak": byts / d["s_per_step"] / 1e9 / HBM_PEAK_GBS, "family_ms": {n: round(v, 4) for n, v in zip(SERVE_FAMILIES, d["family_ms"])},
+                                       "gemm_family_frac_of_hbm_peak": (byts - state) / (d["family_ms"][1] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                       "state_bytes_per_step": state}
+                if nR + nM:
+                    r["decode_b%d" % B]["mixer_family_frac_of_hbm_peak"] = state / (d["family_ms"][3] * 1e-3) / 1e9 / HBM_PEAK_GBS
+            res["midisun_" + label] = r
+            del eng; gc.collect()
+        # ---------------- Lomutar at the same sizes (windowed attention with a sink, rotation, group-limited router, clamped experts + shared expert)
+        layers = [S.LayerSpec(heads=H, kv_heads=G, dim=D, vdim=D, rot_dims=D // 2, rot_base=1e6, rot_factor=2.0, qk_unit_norm=1, scale=D ** -0.5, window=z["window"], has_sink=1,
+                              mlp_kind=S.MLP_MOE, experts=E, top=k, groups=4, keep=2, expert_ff=F, expert_limit=7.0, shared_ff=F, shared_limit=7.0) for _ in range(L)]
+        eng = SCH.BatchEngine(R.ServeModelSpec(V, W, S.NORM_LAYER, 1e-5, layers, None), dtype="bfloat16", max_tokens=4 * (P + 256), max_slots=4)
+        eng.load_synthetic(seed=7, amp=1.0)
+        m = serve_measure(eng, V, P, np.random.default_rng(3))
+        w_att_lo = (H * D + 2 * G * D) * W + W * H * D
+        macs_tok = L * (w_att_lo + (k + 1) * 3 * W * F + E * W)
+        fam = m["prefill_family_ms"]
+        r = {"prefill": {"tok_s": P / m["prefill_s"], "ms": m["prefill_s"] * 1e3, "tokens": P, "family_ms": {n: round(v, 3) for n, v in zip(SERVE_FAMILIES, fam)},
+                         "gemm_family_frac_of_bf16_peak": 2.0 * P * (macs_tok + V * W / P) / (fam[1] * 1e-3) / 1e12 / F16_PEAK_TFLOPS,
+                         "mixer_family_TFLOPs": L * att_flops / (fam[3] * 1e-3) / 1e12}}
+        r["prefill"]["mixer_frac_of_f32_peak"] = r["prefill"]["mixer_family_TFLOPs"] / F32_MATRIX_PEAK_TFLOPS
+        for B, d in m["decode"].items():
+            byts = 2.0 * (L * (w_att_lo + (min(E, B * k) + 1) * 3 * W * F + E * W * 2) + V * W)
             r["decode_b%d" % B] = {"tok_s": B / d["s_per_step"], "ms_per_step": d["s_per_step"] * 1e3, "weight_bytes_per_step": byts,
                                    "frac_of_hbm_peak": byts / d["s_per_step"] / 1e9 / HBM_PEAK_GBS, "family_ms": {n: round(v, 4) for n, v in zip(SERVE_FAMILIES, d["family_ms"])},
                                    "gemm_family_frac_of_hbm_peak": byts / (d["family_ms"][1] * 1e-3) / 1e9 / HBM_PEAK_GBS}
@@ -1548,7 +1634,7 @@ def main_multi(args, torch, dist, world, rank, local_rank):
 def main():
     args = parse()
     if args.arch_compare:
-        return arch_compare_pamulix(args) if args.arch_design == "pamulix" else arch_compare(args)
+        return {"pamulix": arch_compare_pamulix, "midisun": arch_compare_midisun}.get(args.arch_design, arch_compare)(args)
     import torch
     import torch.distributed as dist
 

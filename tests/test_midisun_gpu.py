@@ -294,7 +294,7 @@ def test_far_token_among_hundreds_through_the_state(kind):
     toks_moved = list(toks); toks_moved[40] = 5
     ref_moved, _ = O.forward(cfg, W, toks_moved)
     assert rel(ref_moved[740:741], ref[740:741]) > 0.1           # the far token carries the answer
-    eng = engine(cfg, W, max_tokens=832)
+    eng = engine(cfg, W, max_tokens=1024)
     eng.step([("a", toks[:300], []), ("other", toks_moved[:90], [])])
     eng.step([("a", toks[300:700], [])])
     lg, _ = eng.step([("a", toks[700:], [40]), ("other", toks_moved[90:95], [])])

@@ -1,7 +1,8 @@
 """Probe: a layer-described design on the batched serving store at one of bench.py's --arch-compare sizes, random bf16 weights.
     python tools/probes/serve_profile.py <small|large> prefill [design]     three prompt passes of the size's prompt length
     python tools/probes/serve_profile.py <small|large> decode [design]      decode steps of 1 and of 4 requests at the end of such a prompt, graphs on / off
-design: lomutar (default), or pamulix:<one letter per layer, A = chunked attention, L = attention through latents>, e.g. pamulix:ALAA
+design: lomutar (default), pamulix:<one letter per layer, A = chunked attention, L = attention through latents>, e.g. pamulix:ALAA, or
+midisun:<A = windowed attention, R = retention, M = mLSTM>, e.g. midisun:ARMA
 Run under `rocprofv3 --kernel-trace --stats` for the kernel tables in profiles/serve_*."""
 import os
 import sys
@@ -22,6 +23,8 @@ layers = [S.LayerSpec(heads=H, kv_heads=G, dim=D, vdim=D, rot_dims=D // 2, rot_b
                       mlp_kind=S.MLP_MOE, experts=E, top=k, groups=4, keep=2, expert_ff=F, expert_limit=7.0, shared_ff=F, shared_limit=7.0) for _ in range(L)]
 if design.startswith("pamulix:"):
     eng = bench.pamulix_serve_engine(z, design.split(":", 1)[1])
+elif design.startswith("midisun:"):
+    eng = bench.midisun_serve_engine(z, design.split(":", 1)[1])
 else:
     eng = SCH.BatchEngine(R.ServeModelSpec(V, W, S.NORM_LAYER, 1e-5, layers, None), dtype="bfloat16", max_tokens=4 * (P + 256), max_slots=4)
     eng.load_synthetic(seed=7, amp=1.0)
