@@ -63,7 +63,8 @@ struct kr_serve {
     std::vector<int> h_table;
     // step scratch
     DevBuf meta, x, h, qkv, att, mix, gu, y, rows, ffout, ids, wts, rz, moe_i, hw, logits, amax, part_ml, part_acc;
-    DevBuf h32, hc, rg, qk_rms, lin_o;                   // f32 copy of the mixer's normed input, its convolved form, residual gate logits, whole-row q / k statistics, recurrent outputs
+    DevBuf h32, hc, rg, qk_rms, lin_o, lin_tok, lin_sbuf, lin_nbuf;   // ... ; chunked recurrence: per-token gate terms, state / normaliser at every block's start
+    //                                  f32 copy of the mixer's normed input, its convolved form, residual gate logits, whole-row q / k statistics, recurrent outputs
     DevBuf v_first;                                      // [T, kv_heads * vdim] f32: the values of the first value-mixing layer
     DevBuf lq_c, lq_2, lq_n, lq_e, att2, head_i;         // latent mixer: query latent, W_uq output, plain query parts, folded queries, per-head values, head row tables
     void* h_meta = nullptr; size_t h_meta_bytes = 0;     // pinned staging of the per-step arrays
@@ -604,7 +605,7 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
     for (int i = 0; i < n_want; i++) if (want_rows[i] < 0 || want_rows[i] >= T) return kr_fail(KR_ERR_VALUE, "wanted row %d of %d", want_rows[i], T);
     if (need_pages > (int)s->free_pages.size()) return kr_fail(KR_ERR_STATE, "cache pool exhausted: %d pages needed, %zu free", need_pages, s->free_pages.size());
     // ---- per-step arrays: tokens | slot | pos | want | page table
-    const size_t n_meta = (size_t)3 * T + n_want + 2 * (size_t)n_entries + 1;      // ... | first row of every entry and the end | slot of every entry
+    const size_t n_meta = (size_t)3 * T + n_want + 3 * (size_t)n_entries + 2;      // ... | first row of every entry and the end | slot of every entry | first 64-token block of every entry and the end
     const size_t meta_bytes = (n_meta + s->h_table.size()) * 4;
     if (meta_bytes > s->h_meta_bytes) {
         if (s->h_meta) (void)hipHostFree(s->h_meta);
@@ -613,22 +614,22 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         s->h_meta_bytes = meta_bytes * 2;
     }
     int* hm = (int*)s->h_meta;
-    int* h_tok = hm; int* h_slot = hm + T; int* h_pos = hm + 2 * T; int* h_want = hm + 3 * T; int* h_eoff = h_want + n_want; int* h_eslot = h_eoff + n_entries + 1;
+    int* h_tok = hm; int* h_slot = hm + T; int* h_pos = hm + 2 * T; int* h_want = hm + 3 * T; int* h_eoff = h_want + n_want; int* h_eslot = h_eoff + n_entries + 1; int* h_echunk = h_eslot + n_entries;
     int* h_tab = hm + n_meta;
-    int max_pos = 0;
+    int max_pos = 0, n_chunks = 0, max_count = 0;
     {
         int t = 0;
         for (int e = 0; e < n_entries; e++) {
             SvSlot& q = s->slots[slots[e]];
             max_pos = std::max(max_pos, q.len + counts[e] - 1);
-            h_eoff[e] = t; h_eslot[e] = slots[e];
+            h_eoff[e] = t; h_eslot[e] = slots[e]; h_echunk[e] = n_chunks; n_chunks += (counts[e] + 63) / 64; max_count = std::max(max_count, counts[e]);
             const int np = (q.len + counts[e] + PT - 1) / PT;
             while ((int)q.pages.size() < np) { q.pages.push_back(s->free_pages.back()); s->free_pages.pop_back(); }
             for (int i = 0; i < counts[e]; i++, t++) { h_tok[t] = tokens[t]; h_slot[t] = slots[e]; h_pos[t] = q.len + i; }
             for (size_t p = 0; p < q.pages.size(); p++) s->h_table[(size_t)slots[e] * s->n_pages + p] = q.pages[p];
             q.len += counts[e];
         }
-        h_eoff[n_entries] = t;
+        h_eoff[n_entries] = t; h_echunk[n_entries] = n_chunks;
         for (int i = 0; i < n_want; i++) h_want[i] = want_rows[i];
         std::memcpy(h_tab, s->h_table.data(), s->h_table.size() * 4);
     }
@@ -636,15 +637,22 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
     hipStream_t st = s->st;
     KR_HIP(hipMemcpyAsync(s->meta.p, hm, meta_bytes, hipMemcpyHostToDevice, st));
     const int* d_tok = (const int*)s->meta.p; const int* d_slot = d_tok + T; const int* d_pos = d_tok + 2 * T; const int* d_want = d_tok + 3 * T;
-    const int* d_eoff = d_want + n_want; const int* d_eslot = d_eoff + n_entries + 1;
+    const int* d_eoff = d_want + n_want; const int* d_eslot = d_eoff + n_entries + 1; const int* d_echunk = d_eslot + n_entries;
     const int* d_tab = d_tok + n_meta;
     // ---- scratch sized for this step
     const bool seq = c.block_kind == KR_SERVE_BLOCK_SEQUENTIAL;
     size_t max_qkv = 0, max_att = 0, max_gu = 0, max_y = 0, max_rows = 0, max_pairs = 0, max_vf = 0; int max_E = 1;
-    size_t lq_c = 0, lq_2 = 0, lq_n = 0, lq_e = 0, att2 = 0, head_i = 0, max_lin = 0; bool whole_norm = false;
+    size_t lq_c = 0, lq_2 = 0, lq_n = 0, lq_e = 0, att2 = 0, head_i = 0, max_lin = 0, lin_tok = 0, lin_sb = 0, lin_nb = 0; bool whole_norm = false;
+    // prompt portions take the chunked form of the recurrent mixers (blocks of 64 tokens on the matrix instruction), decode-sized steps the token-by-token form
+    const bool lin_chunked = max_count >= 32;
     for (const SvLayer& l : s->L) {
         const kr_serve_layer& d = l.d;
-        if (l.recurrent()) max_lin = std::max(max_lin, (size_t)d.heads * d.vdim);
+        if (l.recurrent()) {
+            max_lin = std::max(max_lin, (size_t)d.heads * d.vdim);
+            if (lin_chunked && kr_sv_lin_chunked_fits(d.dim, d.vdim)) {
+                lin_tok = std::max(lin_tok, (size_t)d.heads); lin_sb = std::max(lin_sb, (size_t)d.heads * d.dim * d.vdim); lin_nb = std::max(lin_nb, (size_t)d.heads * d.dim);
+            }
+        }
         if (d.qk_unit_norm == KR_SERVE_QKNORM_WHOLE) whole_norm = true;
         max_qkv = std::max(max_qkv, (size_t)l.n_h); max_att = std::max(max_att, (size_t)d.heads * l.att_vdim());
         if (d.v_mix) max_vf = std::max(max_vf, (size_t)d.kv_heads * d.vdim);
@@ -670,7 +678,8 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
                     s->att2.ensure(Ts * att2 * s->esz) || s->head_i.ensure((2 * Ts * head_i + head_i + 1) * 4))))
         return kr_fail(KR_ERR_HIP, "mixer scratch for %d tokens", T);
     if ((c.canon_taps > 1 && (s->h32.ensure(Ts * W * 4) || s->hc.ensure(Ts * W * s->esz))) || (c.res_gate && s->rg.ensure(Ts * W * 4)) || (whole_norm && s->qk_rms.ensure(Ts * 2 * 4)) ||
-        (max_lin && s->lin_o.ensure(Ts * max_lin * 4)))
+        (max_lin && s->lin_o.ensure(Ts * max_lin * 4)) ||
+        (lin_tok && (s->lin_tok.ensure(Ts * lin_tok * 16) || s->lin_sbuf.ensure((size_t)n_chunks * lin_sb * 4) || s->lin_nbuf.ensure((size_t)n_chunks * lin_nb * 4))))
         return kr_fail(KR_ERR_HIP, "block scratch for %d tokens", T);
     for (SvRope& r : s->ropes) if (r.cs.ensure(Ts * (r.dims / 2) * 8)) return kr_fail(KR_ERR_HIP, "rope table");
     if (s->capture) { if (s->cap.ensure((size_t)c.n_layers * Ts * W * 4)) return kr_fail(KR_ERR_HIP, "capture buffer"); s->cap_T = T; }
@@ -776,7 +785,8 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
             q.state = (float*)l.lin_state.p; q.state_stride = l.lin_state_stride; q.nm = (float*)l.lin_nm.p; q.nm_stride = l.lin_nm_stride;
             q.ent_off = d_eoff; q.ent_slot = d_eslot; q.n_entries = n_entries; q.pos = d_pos; q.T = T;
             q.o = (float*)s->lin_o.p; q.norm_w = d.lin_norm_weight ? (const float*)l.lin_norm.p : nullptr; q.eps = c.norm_eps; q.out = s->att.p;
-            { Timer tm(s, 3); kr_sv_lin_scan(q, st); }
+            q.ent_chunk0 = d_echunk; q.n_chunks = n_chunks; q.tok = (float4*)s->lin_tok.p; q.sbuf = (float*)s->lin_sbuf.p; q.nbuf = (float*)s->lin_nbuf.p;
+            { Timer tm(s, 3); if (lin_chunked && kr_sv_lin_chunked_fits(d.dim, d.vdim)) kr_sv_lin_chunked(q, st); else kr_sv_lin_scan(q, st); }
             { Timer tm(s, 2); kr_sv_lin_out(q, s->f32, st); }
         } else if (!l.latent()) {
             a.qkv = hz; a.ldq = l.n_h; a.rot_dims = d.rot_dims; a.rot_interleaved = d.rot_interleaved; a.unit_norm = d.qk_unit_norm; a.own_kv = d.kv_from < 0;

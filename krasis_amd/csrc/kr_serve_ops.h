@@ -155,8 +155,19 @@ struct KrSvLin {
     float* o;                        // [T, heads * vdim] f32 scratch
     const float* norm_w; float eps;  // [heads * vdim] or null
     void* out;                       // [T, heads * vdim] storage type
+    // chunked form (prompt portions): blocks of 64 tokens counted from the start of every entry's portion; entry e owns the blocks
+    // [ent_chunk0[e], ent_chunk0[e + 1])
+    const int* ent_chunk0; int n_chunks;
+    float4* tok;                     // [T, heads]: per token (u = F - m, w = b - F, g = exp(F + m_start - m), exp(-m)); F = log decay summed from the block's start
+    float* sbuf; float* nbuf;        // [n_chunks, heads, dim, vdim] / [n_chunks, heads, dim]: state and normaliser at every block's start
 };
+// token by token, the state in registers: decode steps and short portions
 void kr_sv_lin_scan(const KrSvLin& a, hipStream_t st);
+// prompt portions in blocks of 64 tokens on the f32 matrix instruction (rotation and scales applied to q / k in place first): within a block
+// o_t = g_t S_start^T q_t + sum_(s <= t) exp(u_t + w_s) (q_t . k_s) v_s, and S_end = g_last S_start + sum_s exp(u_last + w_s) k_s v_s^T; a short serial
+// launch carries S from block to block, the outputs of all blocks are formed in parallel.  Same state layout as kr_sv_lin_scan.
+bool kr_sv_lin_chunked_fits(int dim, int vdim);
+void kr_sv_lin_chunked(const KrSvLin& a, hipStream_t st);
 void kr_sv_lin_out(const KrSvLin& a, bool f32, hipStream_t st);
 void kr_sv_argmax(const float* logits, int R, int vocab, int* out, hipStream_t st);
 // uniform values in [-amp, amp) from a counter hash of (seed, element); amp = 0 writes zeros

@@ -1075,6 +1075,195 @@ __global__ void __launch_bounds__(64) sv_lin_scan_kernel(const KrSvLin a) {
     if (ML && lane == 0) nmg[dim] = m;
 }
 
+// ---- chunked form for prompt portions (KrSvLin: tok, sbuf, nbuf)
+// rotation and scales on q / k in place, and the log gates of every (token, head): tok.x = log decay a, tok.y = log input b
+__global__ void __launch_bounds__(64) sv_lin_prep_kernel(const KrSvLin a) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, H = a.heads, dim = a.dim;
+    float* q = a.z + (size_t)t * a.ld + (size_t)h * dim; float* k = q + (size_t)H * dim;
+    const int half = a.rot_dims / 2;
+    for (int i = lane; i < half; i += 64) {
+        const float2 c = a.cs[(size_t)t * half + i];
+        const float qu = q[i] * a.q_scale, qv = q[i + half] * a.q_scale, ku = k[i] * a.k_scale, kv = k[i + half] * a.k_scale;
+        q[i] = qu * c.x - qv * c.y; q[i + half] = qv * c.x + qu * c.y;
+        k[i] = ku * c.x - kv * c.y; k[i + half] = kv * c.x + ku * c.y;
+    }
+    for (int d = a.rot_dims + lane; d < dim; d += 64) { q[d] *= a.q_scale; k[d] *= a.k_scale; }
+    if (lane == 0) {
+        float la, lb;
+        if (a.kind == 3) {
+            const float* zg = a.z + (size_t)t * a.ld + (size_t)2 * H * dim + (size_t)2 * H * a.vdim;
+            float zi = zg[h] + a.i_bias[h], zf = zg[H + h] + a.f_bias[h];
+            if (a.gate_cap > 0.0f) { zi = a.gate_cap * tanhf(zi / a.gate_cap); zf = a.gate_cap * tanhf(zf / a.gate_cap); }
+            lb = zi; la = fminf(zf, 0.0f) - log1pf(expf(-fabsf(zf)));
+        } else { la = fmaxf(logf(a.decay[h]), -1.0e4f); lb = 0.0f; }
+        a.tok[(size_t)t * H + h] = make_float4(la, lb, 0.0f, 0.0f);
+    }
+}
+// one wave per (entry, head): per block of 64 tokens the running sum F of the log decays and the running maximum m, both as scans over the lanes:
+// m_t = F_t + max(m_start, max_(s <= t) (b_s - F_s)).  Leaves (F - m, b - F, exp(F + m_start - m), exp(-m)) per token and the last m in the slot's state.
+template <bool ML>
+__global__ void __launch_bounds__(64) sv_lin_mscan_kernel(const KrSvLin a) {
+    const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, H = a.heads, ncb = (a.vdim + 15) / 16;
+    const int t0 = a.ent_off[e], t1 = a.ent_off[e + 1];
+    float* nmh = a.nm + (size_t)a.ent_slot[e] * a.nm_stride + (size_t)h * ncb * (a.dim + 4);
+    float m_run = (ML && a.pos[t0] != 0) ? nmh[a.dim] : 0.0f;
+    for (int c0 = t0; c0 < t1; c0 += 64) {
+        const int t = c0 + lane; const bool ok = t < t1;
+        const float4 ab = ok ? a.tok[(size_t)t * H + h] : make_float4(0.0f, -INFINITY, 0.0f, 0.0f);
+        float F = ab.x;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) { const float up = __shfl_up(F, o); if (lane >= o) F += up; }
+        float4 out;
+        if constexpr (ML) {
+            const float x = ok ? ab.y - F : -INFINITY;
+            float pm = x;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) { const float up = __shfl_up(pm, o); if (lane >= o) pm = fmaxf(pm, up); }
+            const float m = F + fmaxf(m_run, pm);
+            out = make_float4(F - m, x, expf(F + m_run - m), expf(-m));
+            m_run = __shfl(m, min(63, t1 - c0 - 1));
+        } else out = make_float4(F, ok ? -F : -INFINITY, expf(F), 0.0f);
+        if (ok) a.tok[(size_t)t * H + h] = out;
+    }
+    if (ML && lane < ncb) nmh[(size_t)lane * (a.dim + 4) + a.dim] = m_run;
+}
+// serial over the blocks of an entry, one wave per (entry, head, 16 value columns, NDT tiles of 16 key rows): the state tile in the matrix instruction's
+// accumulators (row d = 16 tile + 4 (lane / 16) + i, column = lane % 16); writes the state at every block's start, and the last one into the slot
+template <bool ML, int NDT>
+__global__ void __launch_bounds__(64) sv_lin_cstate_kernel(const KrSvLin a) {
+    const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, r = lane & 15, kq = lane >> 4;
+    const int H = a.heads, dim = a.dim, vdim = a.vdim, ncb = (vdim + 15) / 16;
+    const int cb = blockIdx.z % ncb, dg = blockIdx.z / ncb;
+    const int t0 = a.ent_off[e], t1 = a.ent_off[e + 1], sl = a.ent_slot[e];
+    const bool fresh = a.pos[t0] == 0;
+    const int col = cb * 16 + r; const bool cv = col < vdim;
+    float* Sg = a.state + (size_t)sl * a.state_stride + ((size_t)h * vdim + (cv ? col : 0)) * dim;
+    float* nmg = a.nm + (size_t)sl * a.nm_stride + ((size_t)h * ncb + cb) * (dim + 4);
+    sv_f4 acc[NDT]; float nacc[NDT];
+#pragma unroll
+    for (int x = 0; x < NDT; x++) {
+        const int dt = dg * NDT + x;
+#pragma unroll
+        for (int i = 0; i < 4; i++) { const int d = dt * 16 + 4 * kq + i; acc[x][i] = (!fresh && cv && d < dim) ? Sg[d] : 0.0f; }
+        const int da = dt * 16 + r;
+        nacc[x] = (ML && !fresh && da < dim) ? nmg[da] : 0.0f;
+    }
+    const float* zk = a.z + (size_t)H * dim + (size_t)h * dim; const float* zv = a.z + (size_t)2 * H * dim + (size_t)h * vdim;
+    const int c0 = a.ent_chunk0[e];
+    for (int tb = t0, c = 0; tb < t1; tb += 64, c++) {
+        const int nt = min(64, t1 - tb);
+        const size_t gc = (size_t)(c0 + c) * H + h;
+#pragma unroll
+        for (int x = 0; x < NDT; x++) {
+            const int dt = dg * NDT + x;
+#pragma unroll
+            for (int i = 0; i < 4; i++) { const int d = dt * 16 + 4 * kq + i; if (cv && d < dim) a.sbuf[(gc * dim + d) * vdim + col] = acc[x][i]; }
+            const int da = dt * 16 + r;
+            if (ML && cb == 0 && kq == 0 && da < dim) a.nbuf[gc * dim + da] = nacc[x];
+        }
+        const float4 last = a.tok[(size_t)(tb + nt - 1) * H + h];
+        float nsum[NDT];
+#pragma unroll
+        for (int x = 0; x < NDT; x++) { acc[x] *= last.z; nsum[x] = 0.0f; }
+#pragma unroll 4
+        for (int j = 0; j < 16; j++) {
+            const int s = 4 * j + kq; const size_t ts = (size_t)tb + min(s, nt - 1);
+            const float wgt = s < nt ? expf(last.x + a.tok[ts * H + h].y) : 0.0f;
+            const float bval = cv ? zv[ts * a.ld + col] : 0.0f;
+#pragma unroll
+            for (int x = 0; x < NDT; x++) {
+                const int da = (dg * NDT + x) * 16 + r;
+                const float aval = da < dim ? zk[ts * a.ld + da] * wgt : 0.0f;
+                acc[x] = __builtin_amdgcn_mfma_f32_16x16x4f32(aval, bval, acc[x], 0, 0, 0);
+                nsum[x] += aval;
+            }
+        }
+        if constexpr (ML) {
+#pragma unroll
+            for (int x = 0; x < NDT; x++) { float v = nsum[x]; v += __shfl_xor(v, 16); v += __shfl_xor(v, 32); nacc[x] = __builtin_fmaf(last.z, nacc[x], v); }
+        }
+    }
+#pragma unroll
+    for (int x = 0; x < NDT; x++) {
+        const int dt = dg * NDT + x;
+#pragma unroll
+        for (int i = 0; i < 4; i++) { const int d = dt * 16 + 4 * kq + i; if (cv && d < dim) Sg[d] = acc[x][i]; }
+        const int da = dt * 16 + r;
+        if (ML && kq == 0 && da < dim) nmg[da] = nacc[x];
+    }
+}
+// parallel over blocks: a workgroup per (block, head), wave w owns the 16 tokens [16 w, 16 w + 16) of the block.  As in the matrix-instruction attention both
+// products are formed transposed: S^T[s][t] = K Q^T (queries of the wave's tokens stay in registers: lane (t = lane % 16, quarter = lane / 16) keeps
+// the quarter-th part of q_t), O^T[c][t] += V^T P^T with the weights where the first product left them; the state's share S_start^T q_t goes into the
+// same accumulators first.  DQ >= ceil(dim / 4), DB >= ceil(vdim / 16).
+template <bool ML, int DQ, int DB>
+__global__ void __launch_bounds__(256) sv_lin_cout_kernel(const KrSvLin a) {
+    const int gc = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, kq = lane >> 4;
+    const int H = a.heads, dim = a.dim, vdim = a.vdim, dq = (dim + 3) / 4, nct = (vdim + 15) / 16;
+    int e = 0;
+    while (e + 1 < a.n_entries && a.ent_chunk0[e + 1] <= gc) e++;
+    const int tb = a.ent_off[e] + 64 * (gc - a.ent_chunk0[e]), nt = min(64, a.ent_off[e + 1] - tb);
+    if (wave * 16 >= nt) return;
+    const int trow = wave * 16 + r; const bool tv = trow < nt;
+    const size_t tg = (size_t)tb + min(trow, nt - 1);
+    const float4 me = a.tok[tg * H + h];
+    const float* zq = a.z + (size_t)h * dim; const float* zk = zq + (size_t)H * dim; const float* zv = a.z + (size_t)2 * H * dim + (size_t)h * vdim;
+    float q[DQ];
+#pragma unroll
+    for (int i = 0; i < DQ; i++) { const int d = kq * dq + i; q[i] = (i < dq && d < dim) ? zq[tg * a.ld + d] : 0.0f; }
+    sv_f4 acc[DB];
+#pragma unroll
+    for (int c = 0; c < DB; c++) acc[c] = sv_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    const float* Sc = a.sbuf + ((size_t)gc * H + h) * dim * vdim;
+    float den = 0.0f;
+#pragma unroll 4
+    for (int i = 0; i < DQ; i++) {
+        if (i >= dq) break;
+        const int d = min(kq * dq + i, dim - 1);          // a row past dim meets a zero of q
+#pragma unroll
+        for (int c = 0; c < DB; c++) {
+            if (c < nct) { const int cc = c * 16 + r; acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(cc < vdim ? Sc[(size_t)d * vdim + cc] : 0.0f, q[i], acc[c], 0, 0, 0); }
+        }
+        if constexpr (ML) den = __builtin_fmaf(q[i], a.nbuf[((size_t)gc * H + h) * dim + d], den);
+    }
+    if constexpr (ML) { den += __shfl_xor(den, 16); den += __shfl_xor(den, 32); den *= me.z; }
+#pragma unroll
+    for (int c = 0; c < DB; c++) acc[c] *= me.z;
+    for (int stile = 0; stile <= wave; stile++) {
+        const size_t sg = (size_t)tb + min(stile * 16 + r, nt - 1);
+        sv_f4 st = sv_f4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll 8
+        for (int i = 0; i < DQ; i++) {
+            if (i >= dq) break;
+            st = __builtin_amdgcn_mfma_f32_16x16x4f32(zk[sg * a.ld + min(kq * dq + i, dim - 1)], q[i], st, 0, 0, 0);
+        }
+        float ps = 0.0f;
+        size_t srow[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int s = stile * 16 + 4 * kq + i;
+            srow[i] = (size_t)tb + min(s, nt - 1);
+            const bool ok = tv && s <= trow;
+            const float p = ok ? st[i] * expf(me.x + a.tok[srow[i] * H + h].y) : 0.0f;
+            st[i] = p; ps += p;
+        }
+        if constexpr (ML) { ps += __shfl_xor(ps, 16); ps += __shfl_xor(ps, 32); den += ps; }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int c = 0; c < DB; c++) {
+                if (c < nct) { const int cc = c * 16 + r; acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(cc < vdim ? zv[srow[i] * a.ld + cc] : 0.0f, st[i], acc[c], 0, 0, 0); }
+            }
+    }
+    const float inv = ML ? 1.0f / (fmaxf(fabsf(den), me.w) + 1e-6f) : 1.0f;
+    if (!tv) return;
+    float* o = a.o + tg * H * vdim + (size_t)h * vdim;
+#pragma unroll
+    for (int c = 0; c < DB; c++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) { const int cc = c * 16 + 4 * kq + i; if (c < nct && cc < vdim) o[cc] = acc[c][i] * inv; }
+}
+
 // one wave per (token, head): o / rms(o) (* weight) * act(g) -> the output projection's input
 template <typename T>
 __global__ void __launch_bounds__(64) sv_lin_out_kernel(const KrSvLin a, T* __restrict__ out) {
@@ -1332,6 +1521,24 @@ void kr_sv_lin_scan(const KrSvLin& a, hipStream_t st) {
     if (a.kind == 3) SV_LIN_D(3); else SV_LIN_D(2);
 #undef SV_LIN_D
 #undef SV_LIN
+}
+bool kr_sv_lin_chunked_fits(int dim, int vdim) { return dim <= 128 && vdim <= 128; }
+void kr_sv_lin_chunked(const KrSvLin& a, hipStream_t st) {
+    if (a.T <= 0 || a.n_entries <= 0 || a.n_chunks <= 0) return;
+    const bool ml = a.kind == 3;
+    const int ncb = (a.vdim + 15) / 16, ndt = (a.dim + 15) / 16, ndg = (ndt + 1) / 2;
+    hipLaunchKernelGGL(sv_lin_prep_kernel, dim3(a.T, a.heads), dim3(64), 0, st, a);
+    if (ml) hipLaunchKernelGGL(sv_lin_mscan_kernel<true>, dim3(a.n_entries, a.heads), dim3(64), 0, st, a);
+    else hipLaunchKernelGGL(sv_lin_mscan_kernel<false>, dim3(a.n_entries, a.heads), dim3(64), 0, st, a);
+    const dim3 gs(a.n_entries, a.heads, ncb * ndg);
+    if (ml) hipLaunchKernelGGL((sv_lin_cstate_kernel<true, 2>), gs, dim3(64), 0, st, a);
+    else hipLaunchKernelGGL((sv_lin_cstate_kernel<false, 2>), gs, dim3(64), 0, st, a);
+    const dim3 go(a.n_chunks, a.heads);
+    const bool small = a.dim <= 64 && a.vdim <= 64;
+#define SV_CO(ML_) do { if (small) hipLaunchKernelGGL((sv_lin_cout_kernel<ML_, 16, 4>), go, dim3(256), 0, st, a); \
+                        else hipLaunchKernelGGL((sv_lin_cout_kernel<ML_, 32, 8>), go, dim3(256), 0, st, a); } while (0)
+    if (ml) SV_CO(true); else SV_CO(false);
+#undef SV_CO
 }
 void kr_sv_lin_out(const KrSvLin& a, bool f32, hipStream_t st) {
     if (a.T <= 0) return;
