@@ -1150,8 +1150,26 @@ __global__ void __launch_bounds__(64) sv_lin_cstate_kernel(const KrSvLin a) {
     }
     const float* zk = a.z + (size_t)H * dim + (size_t)h * dim; const float* zv = a.z + (size_t)2 * H * dim + (size_t)h * vdim;
     const int c0 = a.ent_chunk0[e];
-    for (int tb = t0, c = 0; tb < t1; tb += 64, c++) {
+    // a block's operands (16 steps of four tokens: keys of the wave's rows, values of its columns, the tokens' log weights) are requested one block ahead:
+    // nothing of them depends on the state, so the serial chain per block is the products alone
+    float kA[16][NDT], vA[16], wA[16]; float4 lastA;
+    auto fetch = [&](int tb, float (&kk)[16][NDT], float (&vv)[16], float (&ww)[16], float4& last) {
         const int nt = min(64, t1 - tb);
+        last = a.tok[(size_t)(tb + nt - 1) * H + h];
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const int s = 4 * j + kq; const size_t ts = (size_t)tb + min(s, nt - 1);
+            ww[j] = s < nt ? a.tok[ts * H + h].y : -INFINITY;
+            vv[j] = cv ? zv[ts * a.ld + col] : 0.0f;
+#pragma unroll
+            for (int x = 0; x < NDT; x++) { const int da = (dg * NDT + x) * 16 + r; kk[j][x] = da < dim ? zk[ts * a.ld + da] : 0.0f; }
+        }
+    };
+    fetch(t0, kA, vA, wA, lastA);
+    for (int tb = t0, c = 0; tb < t1; tb += 64, c++) {
+        float kB[16][NDT], vB[16], wB[16]; float4 lastB = lastA;
+        const bool more = tb + 64 < t1;
+        if (more) fetch(tb + 64, kB, vB, wB, lastB);
         const size_t gc = (size_t)(c0 + c) * H + h;
 #pragma unroll
         for (int x = 0; x < NDT; x++) {
@@ -1161,26 +1179,31 @@ __global__ void __launch_bounds__(64) sv_lin_cstate_kernel(const KrSvLin a) {
             const int da = dt * 16 + r;
             if (ML && cb == 0 && kq == 0 && da < dim) a.nbuf[gc * dim + da] = nacc[x];
         }
-        const float4 last = a.tok[(size_t)(tb + nt - 1) * H + h];
         float nsum[NDT];
 #pragma unroll
-        for (int x = 0; x < NDT; x++) { acc[x] *= last.z; nsum[x] = 0.0f; }
-#pragma unroll 4
+        for (int x = 0; x < NDT; x++) { acc[x] *= lastA.z; nsum[x] = 0.0f; }
+#pragma unroll
         for (int j = 0; j < 16; j++) {
-            const int s = 4 * j + kq; const size_t ts = (size_t)tb + min(s, nt - 1);
-            const float wgt = s < nt ? expf(last.x + a.tok[ts * H + h].y) : 0.0f;
-            const float bval = cv ? zv[ts * a.ld + col] : 0.0f;
+            const float wgt = expf(lastA.x + wA[j]);             // tokens past the portion's end carry minus infinity
 #pragma unroll
             for (int x = 0; x < NDT; x++) {
-                const int da = (dg * NDT + x) * 16 + r;
-                const float aval = da < dim ? zk[ts * a.ld + da] * wgt : 0.0f;
-                acc[x] = __builtin_amdgcn_mfma_f32_16x16x4f32(aval, bval, acc[x], 0, 0, 0);
+                const float aval = kA[j][x] * wgt;
+                acc[x] = __builtin_amdgcn_mfma_f32_16x16x4f32(aval, vA[j], acc[x], 0, 0, 0);
                 nsum[x] += aval;
             }
         }
         if constexpr (ML) {
 #pragma unroll
-            for (int x = 0; x < NDT; x++) { float v = nsum[x]; v += __shfl_xor(v, 16); v += __shfl_xor(v, 32); nacc[x] = __builtin_fmaf(last.z, nacc[x], v); }
+            for (int x = 0; x < NDT; x++) { float v = nsum[x]; v += __shfl_xor(v, 16); v += __shfl_xor(v, 32); nacc[x] = __builtin_fmaf(lastA.z, nacc[x], v); }
+        }
+        if (more) {
+            lastA = lastB;
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                vA[j] = vB[j]; wA[j] = wB[j];
+#pragma unroll
+                for (int x = 0; x < NDT; x++) kA[j][x] = kB[j][x];
+            }
         }
     }
 #pragma unroll
@@ -1196,47 +1219,56 @@ __global__ void __launch_bounds__(64) sv_lin_cstate_kernel(const KrSvLin a) {
 // products are formed transposed: S^T[s][t] = K Q^T (queries of the wave's tokens stay in registers: lane (t = lane % 16, quarter = lane / 16) keeps
 // the quarter-th part of q_t), O^T[c][t] += V^T P^T with the weights where the first product left them; the state's share S_start^T q_t goes into the
 // same accumulators first.  DQ >= ceil(dim / 4), DB >= ceil(vdim / 16).
-template <bool ML, int DQ, int DB>
+template <bool ML, int DB>
 __global__ void __launch_bounds__(256) sv_lin_cout_kernel(const KrSvLin a) {
+    extern __shared__ __attribute__((aligned(16))) float sl[];      // [32][lds] rows of the block's start state | [4 waves][dq][64] the waves' queries
     const int gc = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, kq = lane >> 4;
     const int H = a.heads, dim = a.dim, vdim = a.vdim, dq = (dim + 3) / 4, nct = (vdim + 15) / 16;
+    const int lds = ((vdim + 31) / 32) * 32 + 16;                   // rows 16 banks apart: the lanes of two neighbouring rows fall into distinct banks
+    float* qs = sl + 32 * lds + (size_t)wave * dq * 64;             // this wave's queries, one word per (step, lane): a register file that loops can index
     int e = 0;
     while (e + 1 < a.n_entries && a.ent_chunk0[e + 1] <= gc) e++;
     const int tb = a.ent_off[e] + 64 * (gc - a.ent_chunk0[e]), nt = min(64, a.ent_off[e + 1] - tb);
-    if (wave * 16 >= nt) return;
+    const bool active = wave * 16 < nt;                             // a wave without tokens still helps to stage the state
     const int trow = wave * 16 + r; const bool tv = trow < nt;
     const size_t tg = (size_t)tb + min(trow, nt - 1);
     const float4 me = a.tok[tg * H + h];
     const float* zq = a.z + (size_t)h * dim; const float* zk = zq + (size_t)H * dim; const float* zv = a.z + (size_t)2 * H * dim + (size_t)h * vdim;
-    float q[DQ];
-#pragma unroll
-    for (int i = 0; i < DQ; i++) { const int d = kq * dq + i; q[i] = (i < dq && d < dim) ? zq[tg * a.ld + d] : 0.0f; }
+    // the reduction index of a matrix instruction is spread over the four 16-lane groups: lane group kq takes the key coordinates d = 4 i + kq
+    for (int i = 0; i < dq; i++) { const int d = 4 * i + kq; qs[i * 64 + lane] = (active && d < dim) ? zq[tg * a.ld + d] : 0.0f; }
     sv_f4 acc[DB];
 #pragma unroll
     for (int c = 0; c < DB; c++) acc[c] = sv_f4{0.0f, 0.0f, 0.0f, 0.0f};
     const float* Sc = a.sbuf + ((size_t)gc * H + h) * dim * vdim;
+    const float* nc = a.nbuf + ((size_t)gc * H + h) * dim;
     float den = 0.0f;
-#pragma unroll 4
-    for (int i = 0; i < DQ; i++) {
-        if (i >= dq) break;
-        const int d = min(kq * dq + i, dim - 1);          // a row past dim meets a zero of q
+    for (int p0 = 0; p0 < dim; p0 += 32) {                          // passes over 32 rows of the state
+        const int rows = min(32, dim - p0);
+        __syncthreads();
+        for (int idx = tid; idx < rows * vdim; idx += 256) { const int rr = idx / vdim, cc = idx - rr * vdim; sl[rr * lds + cc] = Sc[(size_t)(p0 + rr) * vdim + cc]; }
+        __syncthreads();
+        if (active) {
+#pragma unroll 2
+            for (int i = 0; i < 8; i++) {
+                const int lr = 4 * i + kq;
+                const float qi = lr < rows ? qs[(p0 / 4 + i) * 64 + lane] : 0.0f;      // a row past dim meets a zero
+                const float* srow = sl + min(lr, rows - 1) * lds + r;
 #pragma unroll
-        for (int c = 0; c < DB; c++) {
-            if (c < nct) { const int cc = c * 16 + r; acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(cc < vdim ? Sc[(size_t)d * vdim + cc] : 0.0f, q[i], acc[c], 0, 0, 0); }
+                for (int c = 0; c < DB; c++) if (c < nct) acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(c * 16 + r < vdim ? srow[c * 16] : 0.0f, qi, acc[c], 0, 0, 0);
+                if constexpr (ML) den = __builtin_fmaf(qi, nc[min(p0 + lr, dim - 1)], den);
+            }
         }
-        if constexpr (ML) den = __builtin_fmaf(q[i], a.nbuf[((size_t)gc * H + h) * dim + d], den);
     }
+    if (!active) return;
     if constexpr (ML) { den += __shfl_xor(den, 16); den += __shfl_xor(den, 32); den *= me.z; }
 #pragma unroll
     for (int c = 0; c < DB; c++) acc[c] *= me.z;
+#pragma nounroll
     for (int stile = 0; stile <= wave; stile++) {
-        const size_t sg = (size_t)tb + min(stile * 16 + r, nt - 1);
+        const float* krow = zk + ((size_t)tb + min(stile * 16 + r, nt - 1)) * a.ld;
         sv_f4 st = sv_f4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll 8
-        for (int i = 0; i < DQ; i++) {
-            if (i >= dq) break;
-            st = __builtin_amdgcn_mfma_f32_16x16x4f32(zk[sg * a.ld + min(kq * dq + i, dim - 1)], q[i], st, 0, 0, 0);
-        }
+        for (int i = 0; i < dq; i++) st = __builtin_amdgcn_mfma_f32_16x16x4f32(krow[min(4 * i + kq, dim - 1)], qs[i * 64 + lane], st, 0, 0, 0);
         float ps = 0.0f;
         size_t srow[4];
 #pragma unroll
@@ -1535,8 +1567,9 @@ void kr_sv_lin_chunked(const KrSvLin& a, hipStream_t st) {
     else hipLaunchKernelGGL((sv_lin_cstate_kernel<false, 2>), gs, dim3(64), 0, st, a);
     const dim3 go(a.n_chunks, a.heads);
     const bool small = a.dim <= 64 && a.vdim <= 64;
-#define SV_CO(ML_) do { if (small) hipLaunchKernelGGL((sv_lin_cout_kernel<ML_, 16, 4>), go, dim3(256), 0, st, a); \
-                        else hipLaunchKernelGGL((sv_lin_cout_kernel<ML_, 32, 8>), go, dim3(256), 0, st, a); } while (0)
+    const size_t lds = ((size_t)32 * (((a.vdim + 31) / 32) * 32 + 16) + (size_t)4 * ((a.dim + 3) / 4) * 64) * sizeof(float);
+#define SV_CO(ML_) do { if (small) hipLaunchKernelGGL((sv_lin_cout_kernel<ML_, 4>), go, dim3(256), lds, st, a); \
+                        else hipLaunchKernelGGL((sv_lin_cout_kernel<ML_, 8>), go, dim3(256), lds, st, a); } while (0)
     if (ml) SV_CO(true); else SV_CO(false);
 #undef SV_CO
 }
