@@ -1127,92 +1127,93 @@ __global__ void __launch_bounds__(64) sv_lin_mscan_kernel(const KrSvLin a) {
     }
     if (ML && lane < ncb) nmh[(size_t)lane * (a.dim + 4) + a.dim] = m_run;
 }
-// serial over the blocks of an entry, one wave per (entry, head, 16 value columns, NDT tiles of 16 key rows): the state tile in the matrix instruction's
-// accumulators (row d = 16 tile + 4 (lane / 16) + i, column = lane % 16); writes the state at every block's start, and the last one into the slot
+// The state at every block's start, in two launches.  (1) In parallel over the blocks, one wave per (block, head, 16 value columns, NDT tiles of 16 key
+// rows): the block's own contribution U = sum_s exp(u_last + w_s) k_s v_s^T on the matrix instruction (row d = 16 tile + 4 (lane / 16) + i, column =
+// lane % 16), written where the block's start state will stand; the normaliser's contribution sum_s exp(u_last + w_s) k_s likewise.
 template <bool ML, int NDT>
-__global__ void __launch_bounds__(64) sv_lin_cstate_kernel(const KrSvLin a) {
-    const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, r = lane & 15, kq = lane >> 4;
+__global__ void __launch_bounds__(64) sv_lin_cupd_kernel(const KrSvLin a) {
+    const int gcb = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, r = lane & 15, kq = lane >> 4;
     const int H = a.heads, dim = a.dim, vdim = a.vdim, ncb = (vdim + 15) / 16;
     const int cb = blockIdx.z % ncb, dg = blockIdx.z / ncb;
-    const int t0 = a.ent_off[e], t1 = a.ent_off[e + 1], sl = a.ent_slot[e];
-    const bool fresh = a.pos[t0] == 0;
+    int e = 0;
+    while (e + 1 < a.n_entries && a.ent_chunk0[e + 1] <= gcb) e++;
+    const int tb = a.ent_off[e] + 64 * (gcb - a.ent_chunk0[e]), nt = min(64, a.ent_off[e + 1] - tb);
     const int col = cb * 16 + r; const bool cv = col < vdim;
-    float* Sg = a.state + (size_t)sl * a.state_stride + ((size_t)h * vdim + (cv ? col : 0)) * dim;
-    float* nmg = a.nm + (size_t)sl * a.nm_stride + ((size_t)h * ncb + cb) * (dim + 4);
-    sv_f4 acc[NDT]; float nacc[NDT];
-#pragma unroll
-    for (int x = 0; x < NDT; x++) {
-        const int dt = dg * NDT + x;
-#pragma unroll
-        for (int i = 0; i < 4; i++) { const int d = dt * 16 + 4 * kq + i; acc[x][i] = (!fresh && cv && d < dim) ? Sg[d] : 0.0f; }
-        const int da = dt * 16 + r;
-        nacc[x] = (ML && !fresh && da < dim) ? nmg[da] : 0.0f;
-    }
     const float* zk = a.z + (size_t)H * dim + (size_t)h * dim; const float* zv = a.z + (size_t)2 * H * dim + (size_t)h * vdim;
-    const int c0 = a.ent_chunk0[e];
-    // a block's operands (16 steps of four tokens: keys of the wave's rows, values of its columns, the tokens' log weights) are requested one block ahead:
-    // nothing of them depends on the state, so the serial chain per block is the products alone
-    float kA[16][NDT], vA[16], wA[16]; float4 lastA;
-    auto fetch = [&](int tb, float (&kk)[16][NDT], float (&vv)[16], float (&ww)[16], float4& last) {
-        const int nt = min(64, t1 - tb);
-        last = a.tok[(size_t)(tb + nt - 1) * H + h];
+    const float4 last = a.tok[(size_t)(tb + nt - 1) * H + h];
+    float kk[16][NDT], vv[16], ww[16];
 #pragma unroll
-        for (int j = 0; j < 16; j++) {
-            const int s = 4 * j + kq; const size_t ts = (size_t)tb + min(s, nt - 1);
-            ww[j] = s < nt ? a.tok[ts * H + h].y : -INFINITY;
-            vv[j] = cv ? zv[ts * a.ld + col] : 0.0f;
+    for (int j = 0; j < 16; j++) {                                   // every operand of the block is requested before the first product
+        const int s = 4 * j + kq; const size_t ts = (size_t)tb + min(s, nt - 1);
+        ww[j] = s < nt ? a.tok[ts * H + h].y : -INFINITY;            // tokens past the portion's end weigh nothing
+        vv[j] = cv ? zv[ts * a.ld + col] : 0.0f;
 #pragma unroll
-            for (int x = 0; x < NDT; x++) { const int da = (dg * NDT + x) * 16 + r; kk[j][x] = da < dim ? zk[ts * a.ld + da] : 0.0f; }
-        }
-    };
-    fetch(t0, kA, vA, wA, lastA);
-    for (int tb = t0, c = 0; tb < t1; tb += 64, c++) {
-        float kB[16][NDT], vB[16], wB[16]; float4 lastB = lastA;
-        const bool more = tb + 64 < t1;
-        if (more) fetch(tb + 64, kB, vB, wB, lastB);
-        const size_t gc = (size_t)(c0 + c) * H + h;
+        for (int x = 0; x < NDT; x++) { const int da = (dg * NDT + x) * 16 + r; kk[j][x] = da < dim ? zk[ts * a.ld + da] : 0.0f; }
+    }
+    sv_f4 acc[NDT]; float nsum[NDT];
+#pragma unroll
+    for (int x = 0; x < NDT; x++) { acc[x] = sv_f4{0.0f, 0.0f, 0.0f, 0.0f}; nsum[x] = 0.0f; }
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        const float wgt = expf(last.x + ww[j]);
 #pragma unroll
         for (int x = 0; x < NDT; x++) {
-            const int dt = dg * NDT + x;
-#pragma unroll
-            for (int i = 0; i < 4; i++) { const int d = dt * 16 + 4 * kq + i; if (cv && d < dim) a.sbuf[(gc * dim + d) * vdim + col] = acc[x][i]; }
-            const int da = dt * 16 + r;
-            if (ML && cb == 0 && kq == 0 && da < dim) a.nbuf[gc * dim + da] = nacc[x];
-        }
-        float nsum[NDT];
-#pragma unroll
-        for (int x = 0; x < NDT; x++) { acc[x] *= lastA.z; nsum[x] = 0.0f; }
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-            const float wgt = expf(lastA.x + wA[j]);             // tokens past the portion's end carry minus infinity
-#pragma unroll
-            for (int x = 0; x < NDT; x++) {
-                const float aval = kA[j][x] * wgt;
-                acc[x] = __builtin_amdgcn_mfma_f32_16x16x4f32(aval, vA[j], acc[x], 0, 0, 0);
-                nsum[x] += aval;
-            }
-        }
-        if constexpr (ML) {
-#pragma unroll
-            for (int x = 0; x < NDT; x++) { float v = nsum[x]; v += __shfl_xor(v, 16); v += __shfl_xor(v, 32); nacc[x] = __builtin_fmaf(lastA.z, nacc[x], v); }
-        }
-        if (more) {
-            lastA = lastB;
-#pragma unroll
-            for (int j = 0; j < 16; j++) {
-                vA[j] = vB[j]; wA[j] = wB[j];
-#pragma unroll
-                for (int x = 0; x < NDT; x++) kA[j][x] = kB[j][x];
-            }
+            const float aval = kk[j][x] * wgt;
+            acc[x] = __builtin_amdgcn_mfma_f32_16x16x4f32(aval, vv[j], acc[x], 0, 0, 0);
+            nsum[x] += aval;
         }
     }
+    const size_t gc = (size_t)gcb * H + h;
 #pragma unroll
     for (int x = 0; x < NDT; x++) {
         const int dt = dg * NDT + x;
 #pragma unroll
-        for (int i = 0; i < 4; i++) { const int d = dt * 16 + 4 * kq + i; if (cv && d < dim) Sg[d] = acc[x][i]; }
-        const int da = dt * 16 + r;
-        if (ML && kq == 0 && da < dim) nmg[da] = nacc[x];
+        for (int i = 0; i < 4; i++) { const int d = dt * 16 + 4 * kq + i; if (cv && d < dim) a.sbuf[(gc * dim + d) * vdim + col] = acc[x][i]; }
+        if constexpr (ML) {
+            float v = nsum[x]; v += __shfl_xor(v, 16); v += __shfl_xor(v, 32);
+            const int da = dt * 16 + r;
+            if (cb == 0 && kq == 0 && da < dim) a.nbuf[gc * dim + da] = v;
+        }
+    }
+}
+// (2) Serial over the blocks of an entry, but element by element: a thread owns one element of S (or, in the last workgroups of a head, of the
+// normaliser), walks the entry's blocks, leaves the state at the block's start where the block's contribution stood, and takes S <- g_last S + U.
+// The contributions do not depend on the state, so their loads run ahead of the chain.
+template <bool ML>
+__global__ void __launch_bounds__(256) sv_lin_cscan_kernel(const KrSvLin a) {
+    const int e = blockIdx.x, h = blockIdx.y, H = a.heads, dim = a.dim, vdim = a.vdim, ncb = (vdim + 15) / 16;
+    const int t0 = a.ent_off[e], t1 = a.ent_off[e + 1], sl = a.ent_slot[e], c0 = a.ent_chunk0[e], nch = (t1 - t0 + 63) / 64;
+    const bool fresh = a.pos[t0] == 0;
+    const int idx = blockIdx.z * 256 + threadIdx.x;
+    const int nS = dim * vdim;
+    if (idx < nS) {
+        const int d = idx / vdim, col = idx - d * vdim;
+        float* Sg = a.state + (size_t)sl * a.state_stride + ((size_t)h * vdim + col) * dim + d;
+        float S = fresh ? 0.0f : *Sg;
+        float* p = a.sbuf + ((size_t)c0 * H + h) * nS + idx; const size_t step = (size_t)H * nS;
+        int c = 0;
+        for (; c + 4 <= nch; c += 4) {
+            float u[4], g[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) { u[k] = p[(size_t)(c + k) * step]; g[k] = a.tok[(size_t)(min(t0 + 64 * (c + k + 1), t1) - 1) * H + h].z; }
+#pragma unroll
+            for (int k = 0; k < 4; k++) { p[(size_t)(c + k) * step] = S; S = __builtin_fmaf(g[k], S, u[k]); }
+        }
+        for (; c < nch; c++) {
+            const float u = p[(size_t)c * step], g = a.tok[(size_t)(min(t0 + 64 * (c + 1), t1) - 1) * H + h].z;
+            p[(size_t)c * step] = S; S = __builtin_fmaf(g, S, u);
+        }
+        *Sg = S;
+    } else if (ML && idx - nS < dim) {
+        const int d = idx - nS;
+        float* nm = a.nm + (size_t)sl * a.nm_stride + (size_t)h * ncb * (dim + 4);
+        float n = fresh ? 0.0f : nm[d];
+        float* p = a.nbuf + ((size_t)c0 * H + h) * dim + d; const size_t step = (size_t)H * dim;
+        for (int c = 0; c < nch; c++) {
+            const float u = p[(size_t)c * step], g = a.tok[(size_t)(min(t0 + 64 * (c + 1), t1) - 1) * H + h].z;
+            p[(size_t)c * step] = n; n = __builtin_fmaf(g, n, u);
+        }
+        for (int cbk = 0; cbk < ncb; cbk++) nm[(size_t)cbk * (dim + 4) + d] = n;      // every block of value columns keeps its own copy
     }
 }
 // parallel over blocks: a workgroup per (block, head), wave w owns the 16 tokens [16 w, 16 w + 16) of the block.  As in the matrix-instruction attention both
@@ -1254,7 +1255,7 @@ __global__ void __launch_bounds__(256) sv_lin_cout_kernel(const KrSvLin a) {
                 const float qi = lr < rows ? qs[(p0 / 4 + i) * 64 + lane] : 0.0f;      // a row past dim meets a zero
                 const float* srow = sl + min(lr, rows - 1) * lds + r;
 #pragma unroll
-                for (int c = 0; c < DB; c++) if (c < nct) acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(c * 16 + r < vdim ? srow[c * 16] : 0.0f, qi, acc[c], 0, 0, 0);
+                for (int c = 0; c < DB; c++) acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(c * 16 + r < vdim ? srow[c * 16] : 0.0f, qi, acc[c], 0, 0, 0);
                 if constexpr (ML) den = __builtin_fmaf(qi, nc[min(p0 + lr, dim - 1)], den);
             }
         }
@@ -1284,7 +1285,7 @@ __global__ void __launch_bounds__(256) sv_lin_cout_kernel(const KrSvLin a) {
         for (int i = 0; i < 4; i++)
 #pragma unroll
             for (int c = 0; c < DB; c++) {
-                if (c < nct) { const int cc = c * 16 + r; acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(cc < vdim ? zv[srow[i] * a.ld + cc] : 0.0f, st[i], acc[c], 0, 0, 0); }
+                const int cc = c * 16 + r; acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(cc < vdim ? zv[srow[i] * a.ld + cc] : 0.0f, st[i], acc[c], 0, 0, 0);
             }
     }
     const float inv = ML ? 1.0f / (fmaxf(fabsf(den), me.w) + 1e-6f) : 1.0f;
@@ -1562,9 +1563,12 @@ void kr_sv_lin_chunked(const KrSvLin& a, hipStream_t st) {
     hipLaunchKernelGGL(sv_lin_prep_kernel, dim3(a.T, a.heads), dim3(64), 0, st, a);
     if (ml) hipLaunchKernelGGL(sv_lin_mscan_kernel<true>, dim3(a.n_entries, a.heads), dim3(64), 0, st, a);
     else hipLaunchKernelGGL(sv_lin_mscan_kernel<false>, dim3(a.n_entries, a.heads), dim3(64), 0, st, a);
-    const dim3 gs(a.n_entries, a.heads, ncb * ndg);
-    if (ml) hipLaunchKernelGGL((sv_lin_cstate_kernel<true, 2>), gs, dim3(64), 0, st, a);
-    else hipLaunchKernelGGL((sv_lin_cstate_kernel<false, 2>), gs, dim3(64), 0, st, a);
+    const dim3 gu(a.n_chunks, a.heads, ncb * ndg);
+    if (ml) hipLaunchKernelGGL((sv_lin_cupd_kernel<true, 2>), gu, dim3(64), 0, st, a);
+    else hipLaunchKernelGGL((sv_lin_cupd_kernel<false, 2>), gu, dim3(64), 0, st, a);
+    const dim3 gs(a.n_entries, a.heads, (a.dim * a.vdim + (ml ? a.dim : 0) + 255) / 256);
+    if (ml) hipLaunchKernelGGL(sv_lin_cscan_kernel<true>, gs, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(sv_lin_cscan_kernel<false>, gs, dim3(256), 0, st, a);
     const dim3 go(a.n_chunks, a.heads);
     const bool small = a.dim <= 64 && a.vdim <= 64;
     const size_t lds = ((size_t)32 * (((a.vdim + 31) / 32) * 32 + 16) + (size_t)4 * ((a.dim + 3) / 4) * 64) * sizeof(float);
