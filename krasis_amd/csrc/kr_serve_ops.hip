@@ -1107,9 +1107,12 @@ __global__ void __launch_bounds__(64) sv_lin_mscan_kernel(const KrSvLin a) {
     const int t0 = a.ent_off[e], t1 = a.ent_off[e + 1];
     float* nmh = a.nm + (size_t)a.ent_slot[e] * a.nm_stride + (size_t)h * ncb * (a.dim + 4);
     float m_run = (ML && a.pos[t0] != 0) ? nmh[a.dim] : 0.0f;
+    auto gates = [&](int c0) { const int t = c0 + lane; return t < t1 ? a.tok[(size_t)t * H + h] : make_float4(0.0f, -INFINITY, 0.0f, 0.0f); };
+    float4 nxt = gates(t0);
     for (int c0 = t0; c0 < t1; c0 += 64) {
         const int t = c0 + lane; const bool ok = t < t1;
-        const float4 ab = ok ? a.tok[(size_t)t * H + h] : make_float4(0.0f, -INFINITY, 0.0f, 0.0f);
+        const float4 ab = nxt;
+        if (c0 + 64 < t1) nxt = gates(c0 + 64);                  // the next block's gates are on their way during this block's scans
         float F = ab.x;
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) { const float up = __shfl_up(F, o); if (lane >= o) F += up; }
@@ -1268,25 +1271,34 @@ __global__ void __launch_bounds__(256) sv_lin_cout_kernel(const KrSvLin a) {
     for (int stile = 0; stile <= wave; stile++) {
         const float* krow = zk + ((size_t)tb + min(stile * 16 + r, nt - 1)) * a.ld;
         sv_f4 st = sv_f4{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll 8
-        for (int i = 0; i < dq; i++) st = __builtin_amdgcn_mfma_f32_16x16x4f32(krow[min(4 * i + kq, dim - 1)], qs[i * 64 + lane], st, 0, 0, 0);
+        for (int i0 = 0; i0 < dq; i0 += 16) {                    // sixteen key coordinates and queries requested at a time, then their products
+            float kf[16], qf[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) { kf[i] = krow[min(4 * (i0 + i) + kq, dim - 1)]; qf[i] = i0 + i < dq ? qs[(i0 + i) * 64 + lane] : 0.0f; }
+#pragma unroll
+            for (int i = 0; i < 16; i++) st = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[i], qf[i], st, 0, 0, 0);
+        }
         float ps = 0.0f;
         size_t srow[4];
 #pragma unroll
+        for (int i = 0; i < 4; i++) srow[i] = (size_t)tb + min(stile * 16 + 4 * kq + i, nt - 1);
+#pragma unroll
         for (int i = 0; i < 4; i++) {
             const int s = stile * 16 + 4 * kq + i;
-            srow[i] = (size_t)tb + min(s, nt - 1);
             const bool ok = tv && s <= trow;
             const float p = ok ? st[i] * expf(me.x + a.tok[srow[i] * H + h].y) : 0.0f;
             st[i] = p; ps += p;
         }
         if constexpr (ML) { ps += __shfl_xor(ps, 16); ps += __shfl_xor(ps, 32); den += ps; }
+        float vf[4][DB];                                          // the value rows of the tile's keys
 #pragma unroll
         for (int i = 0; i < 4; i++)
 #pragma unroll
-            for (int c = 0; c < DB; c++) {
-                const int cc = c * 16 + r; acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(cc < vdim ? zv[srow[i] * a.ld + cc] : 0.0f, st[i], acc[c], 0, 0, 0);
-            }
+            for (int c = 0; c < DB; c++) { const int cc = c * 16 + r; vf[i][c] = cc < vdim ? zv[srow[i] * a.ld + cc] : 0.0f; }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int c = 0; c < DB; c++) acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[i][c], st[i], acc[c], 0, 0, 0);
     }
     const float inv = ML ? 1.0f / (fmaxf(fabsf(den), me.w) + 1e-6f) : 1.0f;
     if (!tv) return;
