@@ -58,11 +58,11 @@ __global__ void __launch_bounds__(256) sv_embed_kernel(const T* __restrict__ tab
 }
 
 // statistics of `groups` equal consecutive parts of a row (LDS or global): st[2 g] = mean (0 for an RMS norm), st[2 g + 1] = 1 / sqrt(variance + eps).
-// Wave w of the four takes the parts w, w + 4, ...; the caller makes the row visible before and synchronises after.
-template <int KIND>
+// Wave w of the NW takes the parts w, w + NW, ...; the caller makes the row visible before and synchronises after.
+template <int KIND, int NW = 4>
 __device__ __forceinline__ void sv_group_stats(const float* xr, int width, int groups, float eps, float* st) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, gw = width / groups;
-    for (int g = wave; g < groups; g += 4) {
+    for (int g = wave; g < groups; g += NW) {
         const float* xg = xr + (size_t)g * gw;
         float mean = 0.0f;
         if constexpr (KIND == KR_SV_NORM_LAYER) {
@@ -831,10 +831,12 @@ __global__ void sv_act_kernel(const float* __restrict__ gu, int ld, T* __restric
 
 // one workgroup per token: the sublayers' output row is formed in LDS, normed there when the design norms sublayer outputs, gated when the design gates
 // them, added to the residual row, and the new row is written back and handed on in the storage type -- normed for the next sublayer (norm_w) or as it is
-template <typename T, int KIND>
-__global__ void __launch_bounds__(256) sv_residual_norm_kernel(const KrSvResidual a, T* __restrict__ h_out) {
+// NT threads: 256 for prompt-sized steps (many rows), 1024 for decode-sized ones, where a row's workgroup is alone on its compute unit and the
+// per-thread chain of columns is what the launch waits for
+template <typename T, int KIND, int NT>
+__global__ void __launch_bounds__(NT) sv_residual_norm_kernel(const KrSvResidual a, T* __restrict__ h_out) {
     extern __shared__ float xr[];            // [width] | [2 * groups]
-    __shared__ float red[4];
+    __shared__ float red[NT / 64];
     __shared__ int pp_s[64]; __shared__ float w_s[64];      // the token's expert rows and weights, read once (top <= 64; more fall back to global reads)
     const size_t t = blockIdx.x;
     const int width = a.width, top = a.top;
@@ -845,7 +847,7 @@ __global__ void __launch_bounds__(256) sv_residual_norm_kernel(const KrSvResidua
         const int K = a.canon_keep, sl = a.slot[t];
         if ((int)t + K >= a.T || a.slot[t + K] != sl) {
             float* dst = a.canon_state + ((size_t)sl * K + a.pos[t] % K) * width;
-            for (int c = threadIdx.x; c < width; c += 256) dst[c] = a.h32_in[t * width + c];
+            for (int c = threadIdx.x; c < width; c += NT) dst[c] = a.h32_in[t * width + c];
         }
     }
     const bool staged = rows && top <= 64;
@@ -856,7 +858,7 @@ __global__ void __launch_bounds__(256) sv_residual_norm_kernel(const KrSvResidua
         return 1.0f / (1.0f + expf(-z));
     };
     float s1 = 0.0f;
-    for (int c = threadIdx.x; c < width; c += 256) {
+    for (int c = threadIdx.x; c < width; c += NT) {
         const size_t i = t * width + c;
         float ff = 0.0f; bool any = false;
         if (rows) {
@@ -880,16 +882,16 @@ __global__ void __launch_bounds__(256) sv_residual_norm_kernel(const KrSvResidua
     }
     if (a.post_w) {
         float mean = 0.0f, inv = 0.0f;
-        if (a.groups > 1) { __syncthreads(); sv_group_stats<KIND>(xr, width, a.groups, a.eps, gst); __syncthreads(); }
+        if (a.groups > 1) { __syncthreads(); sv_group_stats<KIND, NT / 64>(xr, width, a.groups, a.eps, gst); __syncthreads(); }
         else {
-            if constexpr (KIND == KR_SV_NORM_LAYER) mean = sv_block_sum<4>(s1, red) / (float)width;
+            if constexpr (KIND == KR_SV_NORM_LAYER) mean = sv_block_sum<NT / 64>(s1, red) / (float)width;
             float q = 0.0f;
-            for (int c = threadIdx.x; c < width; c += 256) { const float dv = xr[c] - mean; q = __builtin_fmaf(dv, dv, q); }
-            inv = 1.0f / sqrtf(sv_block_sum<4>(q, red) / (float)width + a.eps);
+            for (int c = threadIdx.x; c < width; c += NT) { const float dv = xr[c] - mean; q = __builtin_fmaf(dv, dv, q); }
+            inv = 1.0f / sqrtf(sv_block_sum<NT / 64>(q, red) / (float)width + a.eps);
         }
         const int gw = a.groups > 1 ? width / a.groups : width;
         s1 = 0.0f;
-        for (int c = threadIdx.x; c < width; c += 256) {
+        for (int c = threadIdx.x; c < width; c += NT) {
             const size_t i = t * width + c;
             if (a.groups > 1) { mean = gst[2 * (c / gw)]; inv = gst[2 * (c / gw) + 1]; }
             float y = (xr[c] - mean) * inv * a.post_w[c];
@@ -901,19 +903,19 @@ __global__ void __launch_bounds__(256) sv_residual_norm_kernel(const KrSvResidua
     }
     if (!h_out) return;
     if (!a.norm_w) {
-        for (int c = threadIdx.x; c < width; c += 256) { sv_st(h_out + t * width + c, xr[c]); if (a.h32_out) a.h32_out[t * width + c] = xr[c]; }
+        for (int c = threadIdx.x; c < width; c += NT) { sv_st(h_out + t * width + c, xr[c]); if (a.h32_out) a.h32_out[t * width + c] = xr[c]; }
         return;
     }
     float mean = 0.0f, inv = 0.0f;
-    if (a.groups > 1) { __syncthreads(); sv_group_stats<KIND>(xr, width, a.groups, a.eps, gst); __syncthreads(); }
+    if (a.groups > 1) { __syncthreads(); sv_group_stats<KIND, NT / 64>(xr, width, a.groups, a.eps, gst); __syncthreads(); }
     else {
-        if constexpr (KIND == KR_SV_NORM_LAYER) mean = sv_block_sum<4>(s1, red) / (float)width;
+        if constexpr (KIND == KR_SV_NORM_LAYER) mean = sv_block_sum<NT / 64>(s1, red) / (float)width;
         float q = 0.0f;
-        for (int c = threadIdx.x; c < width; c += 256) { const float dv = xr[c] - mean; q = __builtin_fmaf(dv, dv, q); }      // a thread re-reads its own columns
-        inv = 1.0f / sqrtf(sv_block_sum<4>(q, red) / (float)width + a.eps);
+        for (int c = threadIdx.x; c < width; c += NT) { const float dv = xr[c] - mean; q = __builtin_fmaf(dv, dv, q); }      // a thread re-reads its own columns
+        inv = 1.0f / sqrtf(sv_block_sum<NT / 64>(q, red) / (float)width + a.eps);
     }
     const int gw = a.groups > 1 ? width / a.groups : width;
-    for (int c = threadIdx.x; c < width; c += 256) {
+    for (int c = threadIdx.x; c < width; c += NT) {
         if (a.groups > 1) { mean = gst[2 * (c / gw)]; inv = gst[2 * (c / gw) + 1]; }
         float v = (xr[c] - mean) * inv * a.norm_w[c];
         if (a.norm_b) v += a.norm_b[c];
@@ -1534,7 +1536,8 @@ void kr_sv_act(const float* gu, int ld, void* y, bool f32, int M, int F, int kin
 void kr_sv_residual_norm(const KrSvResidual& r, bool out_f32, hipStream_t st) {
     if (r.T <= 0) return;
     const size_t lds = (size_t)(r.width + 2 * (r.groups > 1 ? r.groups : 0)) * sizeof(float);
-#define SV_RN(T_, K_) hipLaunchKernelGGL((sv_residual_norm_kernel<T_, K_>), dim3(r.T), dim3(256), lds, st, r, (T_*)r.h_out)
+#define SV_RN(T_, K_) do { if (r.T <= 64) hipLaunchKernelGGL((sv_residual_norm_kernel<T_, K_, 1024>), dim3(r.T), dim3(1024), lds, st, r, (T_*)r.h_out); \
+                        else hipLaunchKernelGGL((sv_residual_norm_kernel<T_, K_, 256>), dim3(r.T), dim3(256), lds, st, r, (T_*)r.h_out); } while (0)
     if (r.kind == KR_SV_NORM_LAYER) { if (out_f32) SV_RN(float, KR_SV_NORM_LAYER); else SV_RN(uint16_t, KR_SV_NORM_LAYER); }
     else { if (out_f32) SV_RN(float, KR_SV_NORM_RMS); else SV_RN(uint16_t, KR_SV_NORM_RMS); }
 #undef SV_RN
