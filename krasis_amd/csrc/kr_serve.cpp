@@ -63,7 +63,7 @@ struct kr_serve {
     std::vector<int> h_table;
     // step scratch
     DevBuf meta, x, h, qkv, att, mix, gu, y, rows, ffout, ids, wts, rz, moe_i, hw, logits, amax, part_ml, part_acc;
-    DevBuf h32, hc, rg, qk_rms, lin_o, lin_tok, lin_sbuf, lin_nbuf;   // ... ; chunked recurrence: per-token gate terms, state / normaliser at every block's start
+    DevBuf h32, hc, rg, qk_rms, lin_o, lin_tok, lin_sbuf, lin_nbuf, lin_cm;   // ... ; chunked recurrence: per-token gate terms, state / normaliser at every block's start
     //                                  f32 copy of the mixer's normed input, its convolved form, residual gate logits, whole-row q / k statistics, recurrent outputs
     DevBuf v_first;                                      // [T, kv_heads * vdim] f32: the values of the first value-mixing layer
     DevBuf lq_c, lq_2, lq_n, lq_e, att2, head_i;         // latent mixer: query latent, W_uq output, plain query parts, folded queries, per-head values, head row tables
@@ -679,7 +679,7 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         return kr_fail(KR_ERR_HIP, "mixer scratch for %d tokens", T);
     if ((c.canon_taps > 1 && (s->h32.ensure(Ts * W * 4) || s->hc.ensure(Ts * W * s->esz))) || (c.res_gate && s->rg.ensure(Ts * W * 4)) || (whole_norm && s->qk_rms.ensure(Ts * 2 * 4)) ||
         (max_lin && s->lin_o.ensure(Ts * max_lin * 4)) ||
-        (lin_tok && (s->lin_tok.ensure(Ts * lin_tok * 16) || s->lin_sbuf.ensure((size_t)n_chunks * lin_sb * 4) || s->lin_nbuf.ensure((size_t)n_chunks * lin_nb * 4))))
+        (lin_tok && (s->lin_tok.ensure(Ts * lin_tok * 16) || s->lin_sbuf.ensure((size_t)n_chunks * lin_sb * 4) || s->lin_nbuf.ensure((size_t)n_chunks * lin_nb * 4) || s->lin_cm.ensure((size_t)n_chunks * lin_tok * 16))))
         return kr_fail(KR_ERR_HIP, "block scratch for %d tokens", T);
     for (SvRope& r : s->ropes) if (r.cs.ensure(Ts * (r.dims / 2) * 8)) return kr_fail(KR_ERR_HIP, "rope table");
     if (s->capture) { if (s->cap.ensure((size_t)c.n_layers * Ts * W * 4)) return kr_fail(KR_ERR_HIP, "capture buffer"); s->cap_T = T; }
@@ -785,7 +785,7 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
             q.state = (float*)l.lin_state.p; q.state_stride = l.lin_state_stride; q.nm = (float*)l.lin_nm.p; q.nm_stride = l.lin_nm_stride;
             q.ent_off = d_eoff; q.ent_slot = d_eslot; q.n_entries = n_entries; q.pos = d_pos; q.T = T;
             q.o = (float*)s->lin_o.p; q.norm_w = d.lin_norm_weight ? (const float*)l.lin_norm.p : nullptr; q.eps = c.norm_eps; q.out = s->att.p;
-            q.ent_chunk0 = d_echunk; q.n_chunks = n_chunks; q.tok = (float4*)s->lin_tok.p; q.sbuf = (float*)s->lin_sbuf.p; q.nbuf = (float*)s->lin_nbuf.p;
+            q.ent_chunk0 = d_echunk; q.n_chunks = n_chunks; q.tok = (float4*)s->lin_tok.p; q.sbuf = (float*)s->lin_sbuf.p; q.nbuf = (float*)s->lin_nbuf.p; q.cmeta = (float*)s->lin_cm.p;
             { Timer tm(s, 3); if (lin_chunked && kr_sv_lin_chunked_fits(d.dim, d.vdim)) kr_sv_lin_chunked(q, st); else kr_sv_lin_scan(q, st); }
             { Timer tm(s, 2); kr_sv_lin_out(q, s->f32, st); }
         } else if (!l.latent()) {

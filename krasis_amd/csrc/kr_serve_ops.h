@@ -160,6 +160,7 @@ struct KrSvLin {
     const int* ent_chunk0; int n_chunks;
     float4* tok;                     // [T, heads]: per token (u = F - m, w = b - F, g = exp(F + m_start - m), exp(-m)); F = log decay summed from the block's start
     float* sbuf; float* nbuf;        // [n_chunks, heads, dim, vdim] / [n_chunks, heads, dim]: state and normaliser at every block's start
+    float* cmeta;                    // [n_chunks, heads, 4]: a block's last F, its last prefix maximum of b - F, the running maximum at its start
 };
 // token by token, the state in registers: decode steps and short portions
 void kr_sv_lin_scan(const KrSvLin& a, hipStream_t st);

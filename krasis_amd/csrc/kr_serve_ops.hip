@@ -1101,36 +1101,59 @@ __global__ void __launch_bounds__(64) sv_lin_prep_kernel(const KrSvLin a) {
         a.tok[(size_t)t * H + h] = make_float4(la, lb, 0.0f, 0.0f);
     }
 }
-// one wave per (entry, head): per block of 64 tokens the running sum F of the log decays and the running maximum m, both as scans over the lanes:
-// m_t = F_t + max(m_start, max_(s <= t) (b_s - F_s)).  Leaves (F - m, b - F, exp(F + m_start - m), exp(-m)) per token and the last m in the slot's state.
+// The running sum F of the log decays (from each block's start) and the running maximum m, m_t = F_t + max(m_start, max_(s <= t) (b_s - F_s)), in three
+// launches: (1) a wave per (block, head) scans F and the prefix maximum of b - F over its 64 lanes, and leaves the block's last values; (2) a thread per
+// (entry, head) carries m from block to block, m_next = F_last + max(m, pm_last), and leaves the last m in the slot's state; (3) a wave per (block, head)
+// forms what the other launches read per token: (F - m, b - F, exp(F + m_start - m), exp(-m)).  Retention (b = 0, no maximum) is done after (1).
 template <bool ML>
-__global__ void __launch_bounds__(64) sv_lin_mscan_kernel(const KrSvLin a) {
-    const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, H = a.heads, ncb = (a.vdim + 15) / 16;
-    const int t0 = a.ent_off[e], t1 = a.ent_off[e + 1];
-    float* nmh = a.nm + (size_t)a.ent_slot[e] * a.nm_stride + (size_t)h * ncb * (a.dim + 4);
-    float m_run = (ML && a.pos[t0] != 0) ? nmh[a.dim] : 0.0f;
-    auto gates = [&](int c0) { const int t = c0 + lane; return t < t1 ? a.tok[(size_t)t * H + h] : make_float4(0.0f, -INFINITY, 0.0f, 0.0f); };
-    float4 nxt = gates(t0);
-    for (int c0 = t0; c0 < t1; c0 += 64) {
-        const int t = c0 + lane; const bool ok = t < t1;
-        const float4 ab = nxt;
-        if (c0 + 64 < t1) nxt = gates(c0 + 64);                  // the next block's gates are on their way during this block's scans
-        float F = ab.x;
+__global__ void __launch_bounds__(64) sv_lin_mlocal_kernel(const KrSvLin a) {
+    const int gc = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, H = a.heads;
+    int e = 0;
+    while (e + 1 < a.n_entries && a.ent_chunk0[e + 1] <= gc) e++;
+    const int tb = a.ent_off[e] + 64 * (gc - a.ent_chunk0[e]), nt = min(64, a.ent_off[e + 1] - tb);
+    const bool ok = lane < nt;
+    const size_t ti = (size_t)(tb + lane) * H + h;
+    const float4 ab = ok ? a.tok[ti] : make_float4(0.0f, -INFINITY, 0.0f, 0.0f);
+    float F = ab.x;
 #pragma unroll
-        for (int o = 1; o < 64; o <<= 1) { const float up = __shfl_up(F, o); if (lane >= o) F += up; }
-        float4 out;
-        if constexpr (ML) {
-            const float x = ok ? ab.y - F : -INFINITY;
-            float pm = x;
+    for (int o = 1; o < 64; o <<= 1) { const float up = __shfl_up(F, o); if (lane >= o) F += up; }
+    if constexpr (!ML) { if (ok) a.tok[ti] = make_float4(F, -F, expf(F), 0.0f); }
+    else {
+        const float x = ok ? ab.y - F : -INFINITY;
+        float pm = x;
 #pragma unroll
-            for (int o = 1; o < 64; o <<= 1) { const float up = __shfl_up(pm, o); if (lane >= o) pm = fmaxf(pm, up); }
-            const float m = F + fmaxf(m_run, pm);
-            out = make_float4(F - m, x, expf(F + m_run - m), expf(-m));
-            m_run = __shfl(m, min(63, t1 - c0 - 1));
-        } else out = make_float4(F, ok ? -F : -INFINITY, expf(F), 0.0f);
-        if (ok) a.tok[(size_t)t * H + h] = out;
+        for (int o = 1; o < 64; o <<= 1) { const float up = __shfl_up(pm, o); if (lane >= o) pm = fmaxf(pm, up); }
+        if (ok) a.tok[ti] = make_float4(F, x, pm, 0.0f);
+        if (lane == nt - 1) { float* cm = a.cmeta + ((size_t)gc * H + h) * 4; cm[0] = F; cm[1] = pm; }
     }
-    if (ML && lane < ncb) nmh[(size_t)lane * (a.dim + 4) + a.dim] = m_run;
+}
+__global__ void __launch_bounds__(64) sv_lin_mchain_kernel(const KrSvLin a) {
+    const int e = blockIdx.x, h = blockIdx.y * 64 + threadIdx.x, H = a.heads, ncb = (a.vdim + 15) / 16;
+    if (h >= H) return;
+    const int t0 = a.ent_off[e], nch = (a.ent_off[e + 1] - t0 + 63) / 64;
+    float* nmh = a.nm + (size_t)a.ent_slot[e] * a.nm_stride + (size_t)h * ncb * (a.dim + 4);
+    float m = a.pos[t0] != 0 ? nmh[a.dim] : 0.0f;
+    float* cm = a.cmeta + ((size_t)a.ent_chunk0[e] * H + h) * 4; const size_t step = (size_t)H * 4;
+    for (int c0 = 0; c0 < nch; c0 += 8) {                        // eight blocks' values are requested together: the chain itself is a few instructions a block
+        float F[8], pm[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) { const size_t o = (size_t)min(c0 + k, nch - 1) * step; F[k] = cm[o]; pm[k] = cm[o + 1]; }
+#pragma unroll
+        for (int k = 0; k < 8; k++) if (c0 + k < nch) { cm[(size_t)(c0 + k) * step + 2] = m; m = F[k] + fmaxf(m, pm[k]); }
+    }
+    for (int cbk = 0; cbk < ncb; cbk++) nmh[(size_t)cbk * (a.dim + 4) + a.dim] = m;
+}
+__global__ void __launch_bounds__(64) sv_lin_mfinal_kernel(const KrSvLin a) {
+    const int gc = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, H = a.heads;
+    int e = 0;
+    while (e + 1 < a.n_entries && a.ent_chunk0[e + 1] <= gc) e++;
+    const int tb = a.ent_off[e] + 64 * (gc - a.ent_chunk0[e]), nt = min(64, a.ent_off[e + 1] - tb);
+    if (lane >= nt) return;
+    const size_t ti = (size_t)(tb + lane) * H + h;
+    const float m0 = a.cmeta[((size_t)gc * H + h) * 4 + 2];
+    const float4 v = a.tok[ti];
+    const float m = v.x + fmaxf(m0, v.z);
+    a.tok[ti] = make_float4(v.x - m, v.y, expf(v.x + m0 - m), expf(-m));
 }
 // The state at every block's start, in two launches.  (1) In parallel over the blocks, one wave per (block, head, 16 value columns, NDT tiles of 16 key
 // rows): the block's own contribution U = sum_s exp(u_last + w_s) k_s v_s^T on the matrix instruction (row d = 16 tile + 4 (lane / 16) + i, column =
@@ -1576,8 +1599,11 @@ void kr_sv_lin_chunked(const KrSvLin& a, hipStream_t st) {
     const bool ml = a.kind == 3;
     const int ncb = (a.vdim + 15) / 16, ndt = (a.dim + 15) / 16, ndg = (ndt + 1) / 2;
     hipLaunchKernelGGL(sv_lin_prep_kernel, dim3(a.T, a.heads), dim3(64), 0, st, a);
-    if (ml) hipLaunchKernelGGL(sv_lin_mscan_kernel<true>, dim3(a.n_entries, a.heads), dim3(64), 0, st, a);
-    else hipLaunchKernelGGL(sv_lin_mscan_kernel<false>, dim3(a.n_entries, a.heads), dim3(64), 0, st, a);
+    if (ml) {
+        hipLaunchKernelGGL(sv_lin_mlocal_kernel<true>, dim3(a.n_chunks, a.heads), dim3(64), 0, st, a);
+        hipLaunchKernelGGL(sv_lin_mchain_kernel, dim3(a.n_entries, (a.heads + 63) / 64), dim3(64), 0, st, a);
+        hipLaunchKernelGGL(sv_lin_mfinal_kernel, dim3(a.n_chunks, a.heads), dim3(64), 0, st, a);
+    } else hipLaunchKernelGGL(sv_lin_mlocal_kernel<false>, dim3(a.n_chunks, a.heads), dim3(64), 0, st, a);
     const dim3 gu(a.n_chunks, a.heads, ncb * ndg);
     if (ml) hipLaunchKernelGGL((sv_lin_cupd_kernel<true, 2>), gu, dim3(64), 0, st, a);
     else hipLaunchKernelGGL((sv_lin_cupd_kernel<false, 2>), gu, dim3(64), 0, st, a);
