@@ -1274,7 +1274,15 @@ __global__ void __launch_bounds__(256) sv_lin_cout_kernel(const KrSvLin a) {
     for (int p0 = 0; p0 < dim; p0 += 32) {                          // passes over 32 rows of the state
         const int rows = min(32, dim - p0);
         __syncthreads();
-        for (int idx = tid; idx < rows * vdim; idx += 256) { const int rr = idx / vdim, cc = idx - rr * vdim; sl[rr * lds + cc] = Sc[(size_t)(p0 + rr) * vdim + cc]; }
+        if ((vdim & 3) == 0) {                                      // 16-byte pieces: sbuf rows and the LDS rows are 16-byte aligned when vdim is a multiple of four
+            const int v4 = vdim >> 2;
+            for (int idx = tid; idx < rows * v4; idx += 256) {
+                const int rr = idx / v4, c4 = idx - rr * v4;
+                *reinterpret_cast<float4*>(sl + rr * lds + 4 * c4) = *reinterpret_cast<const float4*>(Sc + (size_t)(p0 + rr) * vdim + 4 * c4);
+            }
+        } else {
+            for (int idx = tid; idx < rows * vdim; idx += 256) { const int rr = idx / vdim, cc = idx - rr * vdim; sl[rr * lds + cc] = Sc[(size_t)(p0 + rr) * vdim + cc]; }
+        }
         __syncthreads();
         if (active) {
 #pragma unroll 2
@@ -1329,9 +1337,14 @@ __global__ void __launch_bounds__(256) sv_lin_cout_kernel(const KrSvLin a) {
     if (!tv) return;
     float* o = a.o + tg * H * vdim + (size_t)h * vdim;
 #pragma unroll
-    for (int c = 0; c < DB; c++)
+    for (int c = 0; c < DB; c++) {
+        const int c0 = c * 16 + 4 * kq;
+        if ((vdim & 3) == 0) { if (c0 < vdim) *reinterpret_cast<float4*>(o + c0) = make_float4(acc[c][0] * inv, acc[c][1] * inv, acc[c][2] * inv, acc[c][3] * inv); }
+        else {
 #pragma unroll
-        for (int i = 0; i < 4; i++) { const int cc = c * 16 + 4 * kq + i; if (c < nct && cc < vdim) o[cc] = acc[c][i] * inv; }
+            for (int i = 0; i < 4; i++) if (c0 + i < vdim) o[c0 + i] = acc[c][i] * inv;
+        }
+    }
 }
 
 // one wave per (token, head): o / rms(o) (* weight) * act(g) -> the output projection's input
