@@ -1252,7 +1252,7 @@ template <bool ML, int DB>
 __global__ void __launch_bounds__(256) sv_lin_cout_kernel(const KrSvLin a) {
     extern __shared__ __attribute__((aligned(16))) float sl[];      // [32][lds] rows of the block's start state | [4 waves][dq][64] the waves' queries
     const int gc = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, kq = lane >> 4;
-    const int H = a.heads, dim = a.dim, vdim = a.vdim, dq = (dim + 3) / 4, nct = (vdim + 15) / 16;
+    const int H = a.heads, dim = a.dim, vdim = a.vdim, dq = 4 * ((dim + 15) / 16), nct = (vdim + 15) / 16;
     const int lds = ((vdim + 31) / 32) * 32 + 16;                   // rows 16 banks apart: the lanes of two neighbouring rows fall into distinct banks
     float* qs = sl + 32 * lds + (size_t)wave * dq * 64;             // this wave's queries, one word per (step, lane): a register file that loops can index
     int e = 0;
@@ -1263,8 +1263,11 @@ __global__ void __launch_bounds__(256) sv_lin_cout_kernel(const KrSvLin a) {
     const size_t tg = (size_t)tb + min(trow, nt - 1);
     const float4 me = a.tok[tg * H + h];
     const float* zq = a.z + (size_t)h * dim; const float* zk = zq + (size_t)H * dim; const float* zv = a.z + (size_t)2 * H * dim + (size_t)h * vdim;
-    // the reduction index of a matrix instruction is spread over the four 16-lane groups: lane group kq takes the key coordinates d = 4 i + kq
-    for (int i = 0; i < dq; i++) { const int d = 4 * i + kq; qs[i * 64 + lane] = (active && d < dim) ? zq[tg * a.ld + d] : 0.0f; }
+    // the reduction index of a matrix instruction is spread over the four 16-lane groups: in step i lane group kq takes the key coordinate
+    // d = 16 (i / 4) + 4 kq + i % 4, so that four steps of a lane are 16 contiguous bytes of a key row
+    auto dof = [&](int i) { return 16 * (i >> 2) + 4 * kq + (i & 3); };
+    const bool kvec = (a.ld & 3) == 0 && (dim & 15) == 0;          // key rows start 16-byte aligned and hold whole pieces
+    for (int i = 0; i < dq; i++) { const int d = dof(i); qs[i * 64 + lane] = (active && d < dim) ? zq[tg * a.ld + d] : 0.0f; }
     sv_f4 acc[DB];
 #pragma unroll
     for (int c = 0; c < DB; c++) acc[c] = sv_f4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -1287,7 +1290,7 @@ __global__ void __launch_bounds__(256) sv_lin_cout_kernel(const KrSvLin a) {
         if (active) {
 #pragma unroll 2
             for (int i = 0; i < 8; i++) {
-                const int lr = 4 * i + kq;
+                const int lr = dof(i);                            // row inside the pass (a pass is eight steps = 32 rows)
                 const float qi = lr < rows ? qs[(p0 / 4 + i) * 64 + lane] : 0.0f;      // a row past dim meets a zero
                 const float* srow = sl + min(lr, rows - 1) * lds + r;
 #pragma unroll
@@ -1307,7 +1310,17 @@ __global__ void __launch_bounds__(256) sv_lin_cout_kernel(const KrSvLin a) {
         for (int i0 = 0; i0 < dq; i0 += 16) {                    // sixteen key coordinates and queries requested at a time, then their products
             float kf[16], qf[16];
 #pragma unroll
-            for (int i = 0; i < 16; i++) { kf[i] = krow[min(4 * (i0 + i) + kq, dim - 1)]; qf[i] = i0 + i < dq ? qs[(i0 + i) * 64 + lane] : 0.0f; }
+            for (int i = 0; i < 16; i++) qf[i] = i0 + i < dq ? qs[(i0 + i) * 64 + lane] : 0.0f;
+            if (kvec) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float4 k4 = i0 + 4 * j < dq ? *reinterpret_cast<const float4*>(krow + 16 * (i0 / 4 + j) + 4 * kq) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                    kf[4 * j] = k4.x; kf[4 * j + 1] = k4.y; kf[4 * j + 2] = k4.z; kf[4 * j + 3] = k4.w;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; i++) kf[i] = krow[min(dof(i0 + i), dim - 1)];
+            }
 #pragma unroll
             for (int i = 0; i < 16; i++) st = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[i], qf[i], st, 0, 0, 0);
         }
@@ -1625,7 +1638,7 @@ void kr_sv_lin_chunked(const KrSvLin& a, hipStream_t st) {
     else hipLaunchKernelGGL(sv_lin_cscan_kernel<false>, gs, dim3(256), 0, st, a);
     const dim3 go(a.n_chunks, a.heads);
     const bool small = a.dim <= 64 && a.vdim <= 64;
-    const size_t lds = ((size_t)32 * (((a.vdim + 31) / 32) * 32 + 16) + (size_t)4 * ((a.dim + 3) / 4) * 64) * sizeof(float);
+    const size_t lds = ((size_t)32 * (((a.vdim + 31) / 32) * 32 + 16) + (size_t)4 * (4 * ((a.dim + 15) / 16)) * 64) * sizeof(float);
 #define SV_CO(ML_) do { if (small) hipLaunchKernelGGL((sv_lin_cout_kernel<ML_, 4>), go, dim3(256), lds, st, a); \
                         else hipLaunchKernelGGL((sv_lin_cout_kernel<ML_, 8>), go, dim3(256), lds, st, a); } while (0)
     if (ml) SV_CO(true); else SV_CO(false);
