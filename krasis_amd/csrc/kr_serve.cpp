@@ -63,8 +63,9 @@ struct kr_serve {
     std::vector<int> h_table;
     // step scratch
     DevBuf meta, x, h, qkv, att, mix, gu, y, rows, ffout, ids, wts, rz, moe_i, hw, logits, amax, part_ml, part_acc;
-    DevBuf h32, hc, rg, qk_rms, lin_o, lin_tok, lin_sbuf, lin_nbuf, lin_cm;   // ... ; chunked recurrence: per-token gate terms, state / normaliser at every block's start
-    //                                  f32 copy of the mixer's normed input, its convolved form, residual gate logits, whole-row q / k statistics, recurrent outputs
+    // f32 copy of the mixer's normed input, its convolved form, residual gate logits, whole-row q / k statistics, recurrent outputs; chunked recurrence:
+    // per-token gate terms, state / normaliser at every block's start, per-block gate terms
+    DevBuf h32, hc, rg, qk_rms, lin_o, lin_tok, lin_sbuf, lin_nbuf, lin_cm;
     DevBuf v_first;                                      // [T, kv_heads * vdim] f32: the values of the first value-mixing layer
     DevBuf lq_c, lq_2, lq_n, lq_e, att2, head_i;         // latent mixer: query latent, W_uq output, plain query parts, folded queries, per-head values, head row tables
     void* h_meta = nullptr; size_t h_meta_bytes = 0;     // pinned staging of the per-step arrays
