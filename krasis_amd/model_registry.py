@@ -296,8 +296,8 @@ def midisun_spec(cfg: dict) -> ServeModelSpec:
         kind, m = lc.get("type"), lc["mixer"]
         if kind == "attention":
             l = S.LayerSpec(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
-                            qk_unit_norm=S.QKNORM_WHOLE, scale=float(m["scale"]), window=int(m["mask"]["size"]), has_sink=S.SINK_TENSOR, dist_bias=1, dist_bias_exp=8.0,
-                            proj_bias=1, v_from_k=1, softcap=float(m["softcap"]), out_gate=S.OGATE_HEAD_SIGMOID)
+                            qk_unit_norm=S.QKNORM_WHOLE, scale=float(m["scale"]), window=int((m.get("mask") or {}).get("size", 0)), has_sink=S.SINK_TENSOR, dist_bias=1,
+                            dist_bias_exp=8.0, proj_bias=1, v_from_k=1, softcap=float(m.get("softcap") or 0.0), out_gate=S.OGATE_HEAD_SIGMOID)
             if l.vdim != l.dim:
                 raise ValueError(f"layer {i}: the values are the keys, so vdim {l.vdim} must equal dim {l.dim}")
         elif kind == "retention":
@@ -310,7 +310,7 @@ def midisun_spec(cfg: dict) -> ServeModelSpec:
             extra[f"l{i}.mix.decay"] = dec
         elif kind == "mlstm":
             l = S.LayerSpec(heads=int(m["heads"]), kv_heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]), mixer_kind=S.MIX_MLSTM,
-                            gate_cap=float(m["gate_cap"]), lin_norm_weight=1)
+                            gate_cap=float(m.get("gate_cap") or 0.0), lin_norm_weight=1)
         else:
             raise ValueError(f"layer {i}: mixer type {kind!r} is not part of this design")
         mlp = lc.get("mlp")
