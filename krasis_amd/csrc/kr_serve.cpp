@@ -124,7 +124,7 @@ int check_layer(const kr_serve_config& c, const kr_serve_layer* all, int i) {
     const bool rec = d.mixer_kind == KR_SERVE_MIX_RETENTION || d.mixer_kind == KR_SERVE_MIX_MLSTM;
     if (d.mixer_kind != KR_SERVE_MIX_ATTENTION && !lat && !rec) return kr_fail(KR_ERR_VALUE, "layer %d: mixer kind %d", i, d.mixer_kind);
     if (rec) {
-        if (d.kv_heads != d.heads || d.dim > 256) return kr_fail(KR_ERR_VALUE, "layer %d: a recurrent mixer has one key / value head per query head and dim <= 256", i);
+        if (d.kv_heads != d.heads) return kr_fail(KR_ERR_VALUE, "layer %d: a recurrent mixer has one key / value head per query head", i);
         if (d.kv_from >= 0 || d.v_mix || d.qk_unit_norm || d.window || d.chunk || d.has_sink || d.dist_bias || d.proj_bias || d.v_from_k || d.out_gate || d.softcap != 0.0f)
             return kr_fail(KR_ERR_VALUE, "layer %d: an attention-only mechanism is switched on for a recurrent mixer", i);
         if (d.rot_dims && (d.rot_interleaved || d.mixer_kind != KR_SERVE_MIX_RETENTION)) return kr_fail(KR_ERR_VALUE, "layer %d: recurrent mixers rotate half-split pairs, retention only", i);

@@ -1614,7 +1614,7 @@ void kr_sv_lin_scan(const KrSvLin& a, hipStream_t st) {
     const dim3 grid(a.n_entries, a.heads, (a.vdim + 15) / 16);
     const size_t lds = (size_t)(2 * 8 * 4 * dpr + 8 * 16 + 8 * 2) * sizeof(float);
 #define SV_LIN(K_, DP_) hipLaunchKernelGGL((sv_lin_scan_kernel<K_, DP_>), grid, dim3(64), lds, st, a)
-#define SV_LIN_D(K_) do { if (dpr <= 8) SV_LIN(K_, 8); else if (dpr <= 16) SV_LIN(K_, 16); else if (dpr <= 32) SV_LIN(K_, 32); else SV_LIN(K_, 64); } while (0)
+#define SV_LIN_D(K_) do { if (dpr <= 8) SV_LIN(K_, 8); else if (dpr <= 16) SV_LIN(K_, 16); else if (dpr <= 32) SV_LIN(K_, 32); else if (dpr <= 64) SV_LIN(K_, 64); else SV_LIN(K_, 128); } while (0)
     if (a.kind == 3) SV_LIN_D(3); else SV_LIN_D(2);
 #undef SV_LIN_D
 #undef SV_LIN

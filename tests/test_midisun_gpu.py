@@ -116,6 +116,8 @@ MECHANISMS = [
     ("retention_partial_rotation_odd_sizes", [O.layer(O.retention(3, 20, 7, [0.7, 0.95, 1.0], rot_dims=6, base=40.0), None)], {}, None),
     ("retention_wide_values", [O.layer(O.retention(1, 8, 72, [0.93], base=100.0), None)], {}, None),
     ("retention_keys_of_200", [O.layer(O.retention(2, 200, 24, [0.96, 0.999], rot_dims=64), None)], {}, None),
+    ("retention_keys_of_400", [O.layer(O.retention(1, 400, 16, [0.97], rot_dims=100), None)], {}, None),
+    ("mlstm_keys_of_300", [O.layer(O.mlstm(1, 300, 20, gate_cap=5.0), None)], {}, None),
     ("mlstm_plain", [O.layer(O.mlstm(2, 16, 16), None)], {}, None),
     ("mlstm_quiet_input_gate", [O.layer(O.mlstm(3, 12, 20, gate_cap=8.0), None)], {}, quiet_input_gate),
     ("mlstm_tight_cap_odd_sizes", [O.layer(O.mlstm(5, 10, 9, gate_cap=0.7), None)], {}, None),
