@@ -371,6 +371,7 @@ typedef struct kr_serve kr_serve;
 #define KR_SERVE_ACT_GELU_TANH 0       /* gelu_tanh(gate) * up */
 #define KR_SERVE_ACT_CLAMPED_SWIGLU 1  /* g = min(gate, limit), u = clamp(up, +-limit): g * sigmoid(alpha g) * (u + 1) */
 #define KR_SERVE_ACT_SILU 2            /* silu(gate) * up */
+#define KR_SERVE_ACT_RELU2 3           /* un-gated: down(relu(up h)^2); the feed-forward has no gate tensor */
 typedef struct {
     int vocab, width, n_layers;
     int dtype;                  /* KR_SERVE_BF16 | KR_SERVE_F32 */
@@ -392,6 +393,12 @@ typedef struct {
     int res_gate;               /* 1: a sublayer's output is multiplied by sigmoid(W h + b) before it joins the stream; h = the sublayer's (normed) input
                                  * before the input convolution; tensors res_gate1 / res_gate1_b (mixer), res_gate2 / res_gate2_b (feed-forward).
                                  * Sequential pre-normed blocks only */
+    float norm_weight_offset;   /* added to the weight of every block norm, the final norm and the embedding norm at upload (1: weights stored around zero) */
+    int embed_norm;             /* 1: the embedding row is normed (tensor embed_norm, same kind and eps as the block norms) and the normed row is the stream */
+    /* > 0: a second table joins the embedding row (unscaled): row (previous token * bigram_mul_prev + token * bigram_mul_cur) mod bigram_buckets of tensor
+     * bigram [bigram_buckets + 1, width]; a request's first token takes the last row.  The previous token is part of a request's state */
+    int bigram_buckets, bigram_mul_prev, bigram_mul_cur;
+    float logit_scale;          /* 0 or 1: the logits as they are; else logits * logit_scale */
 } kr_serve_config;
 typedef struct {
     /* mixer: attention over the paged cache; the feed-forward follows it or runs beside it (kr_serve_config.block_kind) */
@@ -421,23 +428,45 @@ typedef struct {
     int v_mix;                         /* KR_SERVE_VMIX_*: values blended with the values an earlier layer formed for the same token, before they are cached */
     int router_bias;                   /* KR_SERVE_RBIAS_*: bias[expert] joins the logits before everything, or the scores for the choice only */
     /* ---- attention */
-    int proj_bias;                     /* q, k and the output projection carry biases (tensors q_bias, k_bias, o_bias) */
+    int proj_bias;                     /* 1: q, k and the output projection carry biases (tensors q_bias, k_bias, o_bias); 2: v too (v_bias) */
     int v_from_k;                      /* the values are the keys as projected (with their bias, before any norm); no v projection; vdim == dim */
     float softcap;                     /* > 0: score <- softcap * tanh(score / softcap), after the scale, before the distance bias */
     int out_gate;                      /* KR_SERVE_OGATE_*: the mixer's output is gated by a projection of the mixer's input (tensor out_gate) before W_o */
     /* ---- recurrent mixers (KR_SERVE_MIX_RETENTION, KR_SERVE_MIX_MLSTM): a matrix state S [dim, vdim] per head and request slot, f32, carried from
      * token to token; heads x dim queries and keys, heads x vdim values (kv_heads == heads); rotation (rot_*) applies to q and k of a retention layer */
     float gate_cap;                    /* mlstm: gate pre-activations z <- gate_cap * tanh(z / gate_cap) (0 = uncapped) */
-    int lin_norm_weight;               /* the per-head RMS norm of the mixer's output is followed by a weight [heads * vdim] (tensor lin_norm) */
+    int lin_norm_weight;               /* the per-head RMS norm of the mixer's output is followed by a weight (tensor lin_norm): 1 [heads * vdim], 2 [vdim] shared by the heads */
     /* ---- router */
     int router_score;                  /* KR_SERVE_RSCORE_SOFTMAX | KR_SERVE_RSCORE_SIGMOID */
     int group_score;                   /* KR_SERVE_GSCORE_MAX (a group's largest choice score) | KR_SERVE_GSCORE_TOP2 (the sum of its two largest) */
+    /* ---- layers that run more than once, vectors that join the stream */
+    int weights_of;                    /* 0: the layer owns its tensors; else 1 + the earlier layer whose tensors it uses (same description).  Cache pages and
+                                        * state are the layer's own either way: a block of layers run several times is listed once per run */
+    int pre_add;                       /* 1: tensor pre_add [width] (the layer's own, also with weights_of) is added to the stream before the layer's first norm */
+    /* ---- attention, further */
+    int proj_conv;                     /* > 0: q, k and v pass a causal convolution of this many taps over the request's positions, channel by channel, right after the
+                                        * projection and its bias (tensors q_conv, k_conv, v_conv [channels, taps], the last column is the current token's); the
+                                        * last proj_conv - 1 projected rows of a request are part of its state */
+    /* ---- KR_SERVE_MIX_GLA: S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T (q_t dim^(-1/2)); a_t = sigmoid(W_a2 (W_a1 h) + b)^(1 / decay_tau) per key channel
+     * (tensors decay_a1 [decay_rank, width], decay_a2 [heads * dim, decay_rank], decay_a2_b); o rms-normed per head (lin_norm_weight), times silu(W_g h) */
+    int decay_rank; float decay_tau;
+    /* ---- KR_SERVE_MIX_SSD, alone (mixer_kind) or beside an attention mixer on the same input (side_mixer): ssd_heads heads of ssd_vdim channels, state
+     * [ssd_state, ssd_vdim] per head; W_in h = [z | x | B | C | dt] (inner = ssd_heads * ssd_vdim; B, C: ssd_groups * ssd_state each; dt: ssd_heads);
+     * x, B, C pass a causal convolution of ssd_conv taps with a bias, then silu; dt <- softplus(dt + dt_bias);
+     * S_t = exp(-exp(A_log_h) dt) S_(t-1) + dt B_t x_t^T, y_t = S_t^T C_t + D_h x_t (head h reads group h / (ssd_heads / ssd_groups));
+     * y * silu(z), rms-normed in ssd_norm_groups equal parts, times a weight, then its own output projection.
+     * Beside attention the layer's mixer output is mix_scale * attention + side_scale * ssd (0 reads as 1). */
+    int side_mixer;
+    int ssd_heads, ssd_vdim, ssd_state, ssd_groups, ssd_conv, ssd_norm_groups;
+    float mix_scale, side_scale;
 } kr_serve_layer;
 #define KR_SERVE_BLOCK_PARALLEL 0
 #define KR_SERVE_BLOCK_SEQUENTIAL 1
 #define KR_SERVE_MIX_ATTENTION 0
 #define KR_SERVE_MIX_LATENT 1
 #define KR_SERVE_MIX_RETENTION 2       /* S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t; k scaled by dim^(-1/2) after the rotation; o / rms(o) per head, times silu(W_g h) */
+#define KR_SERVE_MIX_GLA 4             /* a decay per key channel, formed from the input through a low-rank projection (fields decay_*) */
+#define KR_SERVE_MIX_SSD 5             /* selective state space with one decay per head and token (fields ssd_*) */
 #define KR_SERVE_MIX_MLSTM 3           /* exponential input gate and sigmoid forget gate in log space with a running maximum m (m_0 = 0), normaliser state n;
                                         * q scaled by dim^(-1/2); o = S^T q / (max(|n.q|, exp(-m)) + 1e-6); o / rms(o) per head, times a weight, times sigmoid(W_g h) */
 #define KR_SERVE_QKNORM_NONE 0
@@ -453,11 +482,14 @@ typedef struct {
 #define KR_SERVE_GSCORE_TOP2 1
 #define KR_SERVE_OGATE_NONE 0
 #define KR_SERVE_OGATE_HEAD_SIGMOID 1  /* one number per head: tensor out_gate [heads, width] */
+#define KR_SERVE_OGATE_ELEM_SIGMOID 2  /* one number per output coordinate: tensor out_gate [heads * vdim, width] */
 #define KR_SERVE_SINK_NONE 0
 #define KR_SERVE_SINK_TENSOR 1         /* learned score per head */
 #define KR_SERVE_SINK_ZERO 2           /* score 0: one added to the denominator */
 #define KR_SERVE_ROT_LINEAR 0
 #define KR_SERVE_ROT_BY_PARTS 1
+#define KR_SERVE_ROT_BANDS 2           /* by wavelength l = 2 pi / f: l < rot_original / rot_fast keeps f; l > rot_original / rot_slow takes f / rot_factor;
+                                        * between, with s = (rot_original / l - rot_slow) / (rot_fast - rot_slow): (1 - s) f / rot_factor + s f */
 #define KR_SERVE_VMIX_NONE 0
 #define KR_SERVE_VMIX_FIRST 1          /* this layer's values are kept for the later mixing layers of the step */
 #define KR_SERVE_VMIX_BLEND 2          /* v <- (1 - l) v + l v_first, l = tensor vmix */
@@ -474,9 +506,12 @@ enum { KR_SV_EMBED = 0, KR_SV_FINAL_NORM_W, KR_SV_FINAL_NORM_B, KR_SV_HEAD, KR_S
        KR_SV_OUT_GATE,                 /* attention: [heads, width]; recurrent mixers: [heads * vdim, width] */
        KR_SV_CANON, KR_SV_RES_GATE1, KR_SV_RES_GATE1_B, KR_SV_RES_GATE2, KR_SV_RES_GATE2_B,
        KR_SV_LIN_NORM, KR_SV_LIN_DECAY /* [heads] f32, retention */, KR_SV_IGATE, KR_SV_IGATE_B, KR_SV_FGATE, KR_SV_FGATE_B,     /* recurrent mixers */
+       KR_SV_EMBED_NORM, KR_SV_BIGRAM /* layer = -1 */, KR_SV_PRE_ADD, KR_SV_V_BIAS, KR_SV_Q_CONV, KR_SV_K_CONV, KR_SV_V_CONV,
+       KR_SV_DECAY_A1, KR_SV_DECAY_A2, KR_SV_DECAY_A2_B,
+       KR_SV_SSD_IN, KR_SV_SSD_CONV, KR_SV_SSD_CONV_B, KR_SV_SSD_DT_BIAS, KR_SV_SSD_A_LOG, KR_SV_SSD_D, KR_SV_SSD_NORM, KR_SV_SSD_O,
        KR_SV_N_ROLES };
 /* layout version of kr_serve_config / kr_serve_layer: a caller built against another one must not use the library */
-#define KR_SERVE_ABI 3
+#define KR_SERVE_ABI 4
 int kr_serve_abi(void);
 int kr_serve_create(int device_ordinal, const kr_serve_config* cfg, const kr_serve_layer* layers, kr_serve** out);
 void kr_serve_destroy(kr_serve* s);
@@ -504,7 +539,7 @@ int kr_serve_set_capture(kr_serve* s, int enable);
 int kr_serve_read_capture(kr_serve* s, float* out_host, size_t n_floats);
 size_t kr_serve_device_bytes(const kr_serve* s);
 /* measurement hook: HIP-event time of every kernel family over the steps since the last reset (ms), families: 0 norm 1 gemm 2 qk_prep 3 attention 4 router+sort
- * 5 activation 6 residual 7 embed / head rows / argmax */
+ * 5 activation 6 residual 7 embed / head rows / argmax.  Recurrent scans and the short convolutions count as 3 and 2 */
 int kr_serve_set_profiling(kr_serve* s, int enable);
 int kr_serve_get_profile(kr_serve* s, double* ms_by_family, int n);
 

@@ -49,7 +49,9 @@ class ServeConfigC(C.Structure):
     _fields_ = [("vocab", C.c_int), ("width", C.c_int), ("n_layers", C.c_int), ("dtype", C.c_int), ("norm_kind", C.c_int), ("norm_eps", C.c_float),
                 ("max_slots", C.c_int), ("page_tokens", C.c_int), ("pool_tokens", C.c_int),
                 ("block_kind", C.c_int), ("pre_norm", C.c_int), ("post_norm", C.c_int), ("norm_bias", C.c_int), ("residual_mult", C.c_float),
-                ("norm_groups", C.c_int), ("embed_scale", C.c_float), ("canon_taps", C.c_int), ("res_gate", C.c_int)]
+                ("norm_groups", C.c_int), ("embed_scale", C.c_float), ("canon_taps", C.c_int), ("res_gate", C.c_int),
+                ("norm_weight_offset", C.c_float), ("embed_norm", C.c_int), ("bigram_buckets", C.c_int), ("bigram_mul_prev", C.c_int), ("bigram_mul_cur", C.c_int),
+                ("logit_scale", C.c_float)]
 
 
 class ServeLayerC(C.Structure):
@@ -61,10 +63,13 @@ class ServeLayerC(C.Structure):
                 ("mixer_kind", C.c_int), ("q_rank", C.c_int), ("kv_rank", C.c_int), ("rot_scaling", C.c_int), ("rot_original", C.c_double), ("rot_fast", C.c_double),
                 ("rot_slow", C.c_double), ("chunk", C.c_int), ("dist_bias", C.c_int), ("dist_bias_exp", C.c_float), ("v_mix", C.c_int), ("router_bias", C.c_int),
                 ("proj_bias", C.c_int), ("v_from_k", C.c_int), ("softcap", C.c_float), ("out_gate", C.c_int), ("gate_cap", C.c_float), ("lin_norm_weight", C.c_int),
-                ("router_score", C.c_int), ("group_score", C.c_int)]
+                ("router_score", C.c_int), ("group_score", C.c_int),
+                ("weights_of", C.c_int), ("pre_add", C.c_int), ("proj_conv", C.c_int), ("decay_rank", C.c_int), ("decay_tau", C.c_float), ("side_mixer", C.c_int),
+                ("ssd_heads", C.c_int), ("ssd_vdim", C.c_int), ("ssd_state", C.c_int), ("ssd_groups", C.c_int), ("ssd_conv", C.c_int), ("ssd_norm_groups", C.c_int),
+                ("mix_scale", C.c_float), ("side_scale", C.c_float)]
 
 
-SERVE_ABI = 3      # layout version of the two structures above (KR_SERVE_ABI in include/krasis_hip.h)
+SERVE_ABI = 4      # layout version of the two structures above (KR_SERVE_ABI in include/krasis_hip.h)
 
 
 _lib = None

@@ -41,6 +41,7 @@ __device__ __forceinline__ bool gm_find_tile(const int* seg, int n_groups, int t
 
 // ---------------------------------------------------------------------------------------------------------------- small M
 __device__ __forceinline__ float gm_act(float g, float u, int kind, float limit, float alpha) {
+    if (kind == KR_SV_ACT_RELU2) { g = fmaxf(g, 0.0f); return g * g; }
     if (kind == KR_SV_ACT_GELU_TANH) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
     if (kind == KR_SV_ACT_CLAMPED_SWIGLU) { g = fminf(g, limit); u = fminf(fmaxf(u, -limit), limit); return g / (1.0f + expf(-alpha * g)) * (u + 1.0f); }
     return g / (1.0f + expf(-g)) * u;
@@ -70,6 +71,7 @@ __global__ void __launch_bounds__(256) sv_gemv_kernel(const KrSvGemm g, int mbas
         ar[m] = ACT ? nullptr : (const T*)g.A + (size_t)src * g.lda;
         gr[m] = ACT ? g.act_gu + (size_t)src * g.act_ld : nullptr;
     }
+    const int uoff = g.act_kind == KR_SV_ACT_RELU2 ? 0 : g.K;     // an un-gated activation has no up columns: the second read repeats the first
     float acc[MB][CN];
 #pragma unroll
     for (int m = 0; m < MB; m++)
@@ -89,7 +91,7 @@ __global__ void __launch_bounds__(256) sv_gemv_kernel(const KrSvGemm g, int mbas
                     if constexpr (ACT) {
 #pragma unroll
                         for (int q = 0; q < VEC / 4; q++) {
-                            const float4 gg = *reinterpret_cast<const float4*>(gr[m] + k + 4 * q), uu = *reinterpret_cast<const float4*>(gr[m] + g.K + k + 4 * q);
+                            const float4 gg = *reinterpret_cast<const float4*>(gr[m] + k + 4 * q), uu = *reinterpret_cast<const float4*>(gr[m] + uoff + k + 4 * q);
                             af[4 * q] = gm_round<T>(gm_act(gg.x, uu.x, g.act_kind, g.act_limit, g.act_alpha)); af[4 * q + 1] = gm_round<T>(gm_act(gg.y, uu.y, g.act_kind, g.act_limit, g.act_alpha));
                             af[4 * q + 2] = gm_round<T>(gm_act(gg.z, uu.z, g.act_kind, g.act_limit, g.act_alpha)); af[4 * q + 3] = gm_round<T>(gm_act(gg.w, uu.w, g.act_kind, g.act_limit, g.act_alpha));
                         }
@@ -128,7 +130,7 @@ __global__ void __launch_bounds__(256) sv_gemv_kernel(const KrSvGemm g, int mbas
             for (int m = 0; m < MB; m++) {
                 if (m < mcnt) {
                     float av;
-                    if constexpr (ACT) av = gm_round<T>(gm_act(gr[m][k], gr[m][g.K + k], g.act_kind, g.act_limit, g.act_alpha));
+                    if constexpr (ACT) av = gm_round<T>(gm_act(gr[m][k], gr[m][uoff + k], g.act_kind, g.act_limit, g.act_alpha));
                     else av = gm_ld(ar[m] + k);
 #pragma unroll
                     for (int c = 0; c < CN; c++) acc[m][c] = __builtin_fmaf(av, w[c], acc[m][c]);

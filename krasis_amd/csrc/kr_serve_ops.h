@@ -29,11 +29,35 @@ void kr_sv_gemm(const KrSvGemm& g, bool f32, hipStream_t st);
 bool kr_sv_gemm_small(const KrSvGemm& g);      // true: kr_sv_gemm takes the wave-per-column form for this problem (and honours act_gu)
 
 enum { KR_SV_NORM_LAYER = 0, KR_SV_NORM_RMS = 1 };
-enum { KR_SV_ACT_GELU_TANH = 0, KR_SV_ACT_CLAMPED_SWIGLU = 1, KR_SV_ACT_SILU = 2 };
+enum { KR_SV_ACT_GELU_TANH = 0, KR_SV_ACT_CLAMPED_SWIGLU = 1, KR_SV_ACT_SILU = 2, KR_SV_ACT_RELU2 = 3 /* un-gated: relu(x)^2 of the first F columns; no up columns */ };
 
 // x[t] = table[tokens[t]]; with h_out also the row in the storage type (the first sublayer's input in a design without input norms)
 // scale: the row is multiplied by it (1 = as it is)
-void kr_sv_embed(const void* table, bool f32, const int* tokens, float* x, void* h_out, int T, int width, float scale, hipStream_t st);
+// table2 / rows2: optional second table whose row rows2[t] is added as it is (a hashed pair-of-tokens embedding)
+void kr_sv_embed(const void* table, bool f32, const int* tokens, float* x, void* h_out, int T, int width, float scale, const void* table2, const int* rows2, hipStream_t st);
+// the stream itself: x[t] += add (optional [width]); then, with w, either x[t] <- norm(x[t]) * w (in_place: the normed row IS the stream) or
+// out[t] = norm(x[t]) * w in the storage type (the next sublayer's input).  One workgroup per row, the row held in LDS.
+void kr_sv_stream_norm(float* x, const float* add, const float* w, const float* b, bool in_place, void* out, bool out_f32, int T, int width, float eps, int kind, int groups,
+                       hipStream_t st);
+// Short causal convolution over a request's positions on C channels of a projection's output:
+//   y[t][c] = act(cb[c] + sum_j w[c][j] u(position(t) - taps + 1 + j)[c]),  u = in + in_bias, zeros before position 0.
+// u of a position comes from this step's rows when the request's portion holds it, else from the request's ring state[slot][position % (taps - 1)][C];
+// kr_sv_chan_conv_save (a launch of its own, after the convolution has read the ring) keeps the last taps - 1 rows u of every portion.
+struct KrSvChanConv {
+    const float* in; int ld_in;      // [T, ld_in] f32, the C channels start at `in`
+    const float* in_bias;            // [C] or null: joins the input before the convolution (a projection's bias)
+    const float* w; int taps;        // [C, taps] f32, the last column is the current token's
+    const float* cb;                 // [C] or null: the convolution's own bias
+    int act;                         // 0 none, 1 silu
+    float* out; int ld_out;          // [T, ld_out] f32 (not `in`)
+    float* state;                    // [slots][taps - 1][C]
+    const int* slot; const int* pos; int T, C;
+    const int* ent_off; int n_entries;
+};
+void kr_sv_chan_conv(const KrSvChanConv& c, hipStream_t st);
+void kr_sv_chan_conv_save(const KrSvChanConv& c, hipStream_t st);
+// logits <- logits * scale
+void kr_sv_scale(float* p, size_t n, float scale, hipStream_t st);
 // out[r] = norm(x[rows ? rows[r] : r]) * w (+ b): two passes over the row, f32; out in the storage type.  groups > 1: the row is normed in that many equal
 // consecutive parts, each by its own statistics.  out32: optional f32 copy of the normed row (the input of a convolution over positions)
 void kr_sv_norm(const float* x, const int* rows, const float* w, const float* b, void* out, bool out_f32, int R, int width, float eps, int kind, int groups, float* out32,
@@ -68,6 +92,10 @@ struct KrSvAttn {
     int v_from_k;                    // the value rows of the cache are the key rows before their norm (no v block in qkv)
     float softcap;                   // > 0: score <- softcap * tanh(score / softcap) before the distance bias
     const float* out_gate; int ld_gate;   // [T, ld_gate] f32 or null: head h's output is multiplied by sigmoid(out_gate[t][h])
+    const float* v_bias;             // [kv_heads * vdim] or null: joins the values before they are cached
+    int gate_elem;                   // out_gate holds one logit per output coordinate ([T, ld_gate] with heads * vdim columns) instead of one per head
+    float out_scale;                 // the output is multiplied by it before it is rounded (0 reads as 1)
+    int out_ld;                      // row stride of `out` in elements (0: heads * vdim) -- the output may be the leading columns of a wider row
     const float* sink;               // [heads] or null
     const float2* cs;                // rope table of the step for this layer's rotation
     void* kpool; void* vpool;        // [pages][page_tokens][ldk | ldv] storage type; head g at g * dim | g * vdim of a row (vpool may be kpool: values that are a
@@ -141,8 +169,16 @@ void kr_sv_head_rows(int T, int heads, int* seg, int* rows, int* group, hipStrea
 // The state of request slot s: S at state + s * state_stride as [heads][vdim][dim]; normaliser and maximum at nm + s * nm_stride as
 // [heads][vdim blocks of 16][dim + 4] (every block of value columns keeps its own copy, so no two workgroups share a word).  A portion that starts at
 // position 0 starts from zeros whatever the slot held.
+//   gla (4):   S_t = diag(a_t) S_(t-1) + k_t v_t^T, a_t = exp(log sigmoid(gz_t + gz_bias) * inv_tau) per key channel (gz [T, gz_ld], heads x dim)
+//   ssd (5):   S_t = exp(-exp(a_log_h) dt_t) S_(t-1) + dt_t k_t v_t^T with dt_t = softplus(dtz_t[h] + dt_bias[h]); q, k of head h are those of group
+//              h / qk_group (C and B), v the head's x; the skip term and everything after it belong to kr_sv_ssd_out
+// Kinds 4 and 5 read q, k, v through qsrc / ksrc / vsrc (rows src_ld floats apart); the scan form only.
 struct KrSvLin {
-    int kind;                        // KR_SERVE_MIX_RETENTION (2) | KR_SERVE_MIX_MLSTM (3)
+    int kind;                        // KR_SERVE_MIX_RETENTION (2) | KR_SERVE_MIX_MLSTM (3) | KR_SERVE_MIX_GLA (4) | KR_SERVE_MIX_SSD (5)
+    const float* qsrc; const float* ksrc; const float* vsrc; int src_ld, qk_group;      // kinds 4, 5
+    const float* gz; int gz_ld; const float* gz_bias; float inv_tau;                     // kind 4
+    const float* dtz; int dtz_ld; const float* dt_bias; const float* a_log;              // kind 5
+    int norm_shared;                 // norm_w is [vdim], shared by the heads
     float* z; int ld;                // [T, ld] f32: q [heads * dim] | k [heads * dim] | v [heads * vdim] | g [heads * vdim] | (mlstm) z_i [heads] | z_f [heads]
     int heads, dim, vdim, rot_dims;
     const float2* cs;                // rotation table of the step [T, rot_dims / 2] (pairs (i, i + rot_dims / 2))
@@ -170,6 +206,18 @@ void kr_sv_lin_scan(const KrSvLin& a, hipStream_t st);
 bool kr_sv_lin_chunked_fits(int dim, int vdim);
 void kr_sv_lin_chunked(const KrSvLin& a, hipStream_t st);
 void kr_sv_lin_out(const KrSvLin& a, bool f32, hipStream_t st);
+// the selective state-space mixer after its scan: y = (o + D_h x) * silu(z), rms-normed in `groups` equal parts of the inner row, times w, times scale,
+// rounded to the storage type at out[t * out_ld + c]
+struct KrSvSsdOut {
+    const float* o;                  // [T, inner] f32 (the scan's output)
+    const float* x; int ld_x;        // the convolved x rows
+    const float* z; int ld_z;        // the gate's pre-activation
+    const float* D;                  // [heads]
+    const float* w;                  // [inner]
+    int heads, vdim, groups; float eps, scale;
+    void* out; int out_ld; int T;
+};
+void kr_sv_ssd_out(const KrSvSsdOut& a, bool f32, hipStream_t st);
 void kr_sv_argmax(const float* logits, int R, int vocab, int* out, hipStream_t st);
 // uniform values in [-amp, amp) from a counter hash of (seed, element); amp = 0 writes zeros
 void kr_sv_fill_uniform(void* p, bool f32, size_t n, uint64_t seed, float amp, hipStream_t st);

@@ -47,11 +47,13 @@ __device__ __forceinline__ float sv_block_sum(float v, float* red) {
 
 template <typename T>
 __global__ void __launch_bounds__(256) sv_embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens, float* __restrict__ x, T* __restrict__ h_out, int width,
-                                                       float scale) {
+                                                       float scale, const T* __restrict__ table2, const int* __restrict__ rows2) {
     const int t = blockIdx.x;
     const T* row = table + (size_t)tokens[t] * width;
+    const T* row2 = table2 ? table2 + (size_t)rows2[t] * width : nullptr;
     for (int c = threadIdx.x; c < width; c += 256) {
-        const float v = sv_ld(row + c) * scale;
+        float v = sv_ld(row + c) * scale;
+        if (row2) v += sv_ld(row2 + c);
         x[(size_t)t * width + c] = v;
         if (h_out) sv_st(h_out + (size_t)t * width + c, v);
     }
@@ -135,6 +137,73 @@ __global__ void __launch_bounds__(256) sv_canon_kernel(const KrSvCanon a, T* __r
     sv_st(out + (size_t)t * a.width + c, acc);
 }
 
+// the stream itself (kr_sv_stream_norm): a vector joins the row, and / or the row is normed -- in place, or into the next sublayer's input
+template <typename T, int KIND>
+__global__ void __launch_bounds__(256) sv_stream_norm_kernel(float* __restrict__ x, const float* __restrict__ add, const float* __restrict__ w, const float* __restrict__ b, int in_place,
+                                                             T* __restrict__ out, int width, float eps, int groups) {
+    extern __shared__ float xr[];            // [width] | [2 * groups]
+    __shared__ float red[4];
+    const size_t t = blockIdx.x;
+    float* xp = x + t * width;
+    float* gst = xr + width;
+    float s1 = 0.0f;
+    for (int c = threadIdx.x; c < width; c += 256) {
+        float v = xp[c];
+        if (add) { v += add[c]; xp[c] = v; }
+        xr[c] = v; s1 += v;
+    }
+    if (!w) return;
+    float mean = 0.0f, inv = 0.0f;
+    if (groups > 1) { __syncthreads(); sv_group_stats<KIND, 4>(xr, width, groups, eps, gst); __syncthreads(); }
+    else {
+        if constexpr (KIND == KR_SV_NORM_LAYER) mean = sv_block_sum<4>(s1, red) / (float)width;
+        float q = 0.0f;
+        for (int c = threadIdx.x; c < width; c += 256) { const float dv = xr[c] - mean; q = __builtin_fmaf(dv, dv, q); }
+        inv = 1.0f / sqrtf(sv_block_sum<4>(q, red) / (float)width + eps);
+    }
+    const int gw = groups > 1 ? width / groups : width;
+    for (int c = threadIdx.x; c < width; c += 256) {
+        if (groups > 1) { mean = gst[2 * (c / gw)]; inv = gst[2 * (c / gw) + 1]; }
+        float v = (xr[c] - mean) * inv * w[c];
+        if (b) v += b[c];
+        if (in_place) xp[c] = v; else sv_st(out + t * width + c, v);
+    }
+}
+
+// short convolution on the channels of a projection (KrSvChanConv): one thread per (token, channel)
+__global__ void __launch_bounds__(256) sv_chan_conv_kernel(const KrSvChanConv a) {
+    const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= a.C) return;
+    const int p = a.pos[t], sl = a.slot[t], K = a.taps - 1;
+    const float* w = a.w + (size_t)c * a.taps;
+    const float ib = a.in_bias ? a.in_bias[c] : 0.0f;
+    float acc = a.cb ? a.cb[c] : 0.0f;
+    acc = __builtin_fmaf(w[K], a.in[(size_t)t * a.ld_in + c] + ib, acc);
+    for (int d = 1; d <= K; d++) {            // d positions back
+        const int q = p - d;
+        if (q < 0) break;
+        float u;
+        if (t - d >= 0 && a.slot[t - d] == sl) u = a.in[(size_t)(t - d) * a.ld_in + c] + ib;
+        else u = a.state[((size_t)sl * K + q % K) * a.C + c];
+        acc = __builtin_fmaf(w[K - d], u, acc);
+    }
+    if (a.act == 1) acc = acc / (1.0f + expf(-acc));
+    a.out[(size_t)t * a.ld_out + c] = acc;
+}
+// the last taps - 1 inputs of every portion -> the request's ring
+__global__ void __launch_bounds__(256) sv_chan_conv_save_kernel(const KrSvChanConv a) {
+    const int e = blockIdx.x, i = blockIdx.y, c = blockIdx.z * 256 + threadIdx.x, K = a.taps - 1;
+    if (c >= a.C) return;
+    const int t = a.ent_off[e + 1] - 1 - i;
+    if (t < a.ent_off[e]) return;
+    const float ib = a.in_bias ? a.in_bias[c] : 0.0f;
+    a.state[((size_t)a.slot[t] * K + a.pos[t] % K) * a.C + c] = a.in[(size_t)t * a.ld_in + c] + ib;
+}
+__global__ void sv_scale_kernel(float* __restrict__ p, size_t n, float scale) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] *= scale;
+}
+
 // unit_norm == 3: 1 / rms over the whole q row (part 0) and the whole k row (part 1) of every token, biases included
 __global__ void __launch_bounds__(256) sv_qk_rms_kernel(const KrSvAttn a) {
     __shared__ float red[4];
@@ -176,8 +245,9 @@ __global__ void __launch_bounds__(64) sv_qk_prep_kernel(const KrSvAttn a) {
         T* dst = (T*)a.vpool + prow * a.ldv + (size_t)g * a.vdim;
         float* vf = a.v_mix ? a.v_first + ((size_t)t * G + g) * a.vdim : nullptr;
         const float lam = a.v_mix == 2 ? *a.v_lambda : 0.0f;
+        const float* vb = a.v_bias ? a.v_bias + (size_t)g * a.vdim : nullptr;
         for (int d = lane; d < a.vdim; d += 64) {
-            float val = v[d];
+            float val = vb ? v[d] + vb[d] : v[d];
             if (a.v_mix == 1) vf[d] = val;
             else if (a.v_mix == 2) val = (1.0f - lam) * val + lam * vf[d];
             sv_st(dst + d, val);
@@ -448,7 +518,8 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
         }
         __syncthreads();
     }
-    T* o = (T*)a.out + ((size_t)t * a.heads + h0) * vdim;
+    T* o = (T*)a.out + (size_t)t * (a.out_ld ? a.out_ld : a.heads * vdim) + (size_t)h0 * vdim;
+    const float osc = a.out_scale != 0.0f ? a.out_scale : 1.0f;
     for (int i = tid; i < nr * vdim; i += 256) {
         const int r = i / vdim;
         float M = -INFINITY;
@@ -457,8 +528,8 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
         float L = (last && a.sink) ? expf(a.sink[h0 + r] - M) : 0.0f;
         for (int w = 0; w < 4; w++) { const float mw = ml[(w * RM + r) * 2]; if (mw != -INFINITY) L += ml[(w * RM + r) * 2 + 1] * expf(mw - M); }
         if (last) {
-            const float gt = a.out_gate ? 1.0f / (1.0f + expf(-a.out_gate[(size_t)t * a.ld_gate + h0 + r])) : 1.0f;
-            sv_st(o + i, accs[i] / L * gt);
+            const float gt = a.out_gate ? 1.0f / (1.0f + expf(-a.out_gate[(size_t)t * a.ld_gate + (a.gate_elem ? (size_t)h0 * vdim + i : (size_t)(h0 + r))])) : 1.0f;
+            sv_st(o + i, accs[i] / L * gt * osc);
         }
         else {
             const size_t slot = ((size_t)t * a.heads + h0 + r) * a.nsplit + sp;
@@ -652,8 +723,8 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
             const int h = g * R + hb * 16 + (r % Rb);
             const float av = accs[acc_at(r, i - r * vdim)];
             if (last) {
-                const float gt = a.out_gate ? 1.0f / (1.0f + expf(-a.out_gate[(size_t)(t0 + tq) * a.ld_gate + h])) : 1.0f;
-                sv_st((T*)a.out + ((size_t)(t0 + tq) * a.heads + h) * vdim + (i - r * vdim), av * mf[r * 2 + 1] * gt);
+                const float gt = a.out_gate ? 1.0f / (1.0f + expf(-a.out_gate[(size_t)(t0 + tq) * a.ld_gate + (a.gate_elem ? (size_t)h * vdim + (i - r * vdim) : (size_t)h)])) : 1.0f;
+                sv_st((T*)a.out + (size_t)(t0 + tq) * (a.out_ld ? a.out_ld : a.heads * vdim) + (size_t)h * vdim + (i - r * vdim), av * mf[r * 2 + 1] * gt * (a.out_scale != 0.0f ? a.out_scale : 1.0f));
             }
             else {
                 const size_t slot = ((size_t)(t0 + tq) * a.heads + h) * a.nsplit + sp;
@@ -683,12 +754,13 @@ __global__ void __launch_bounds__(256) sv_attn_merge_kernel(const KrSvAttn a) {
         wsp[a.nsplit] = 1.0f / L;
     }
     __syncthreads();
-    const float inv = wsp[a.nsplit] * (a.out_gate ? 1.0f / (1.0f + expf(-a.out_gate[(size_t)t * a.ld_gate + h])) : 1.0f);
-    T* o = (T*)a.out + ((size_t)t * a.heads + h) * a.vdim;
+    const float inv = wsp[a.nsplit] * ((a.out_gate && !a.gate_elem) ? 1.0f / (1.0f + expf(-a.out_gate[(size_t)t * a.ld_gate + h])) : 1.0f) * (a.out_scale != 0.0f ? a.out_scale : 1.0f);
+    T* o = (T*)a.out + (size_t)t * (a.out_ld ? a.out_ld : a.heads * a.vdim) + (size_t)h * a.vdim;
     for (int d = tid; d < a.vdim; d += 256) {
         float v = 0.0f;
 #pragma unroll 8
         for (int s = 0; s < a.nsplit; s++) { const float w = wsp[s], p = a.part_acc[(base + s) * a.vdim + d]; v = __builtin_fmaf(w != 0.0f ? p : 0.0f, w, v); }      // a split without keys counts as zeros
+        if (a.out_gate && a.gate_elem) v *= 1.0f / (1.0f + expf(-a.out_gate[(size_t)t * a.ld_gate + (size_t)h * a.vdim + d]));
         sv_st(o + d, v * inv);
     }
 }
@@ -816,8 +888,10 @@ __global__ void sv_act_kernel(const float* __restrict__ gu, int ld, T* __restric
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (size_t)M * F) return;
     const size_t r = i / F; const int c = (int)(i - r * F);
-    float g = gu[r * ld + c], u = gu[r * ld + F + c], v;
-    if (kind == KR_SV_ACT_GELU_TANH) {
+    float g = gu[r * ld + c], u = kind == KR_SV_ACT_RELU2 ? 0.0f : gu[r * ld + F + c], v;
+    if (kind == KR_SV_ACT_RELU2) {
+        g = fmaxf(g, 0.0f); v = g * g;
+    } else if (kind == KR_SV_ACT_GELU_TANH) {
         const float in = 0.7978845608028654f * (g + 0.044715f * g * g * g);
         v = 0.5f * g * (1.0f + tanhf(in)) * u;
     } else if (kind == KR_SV_ACT_CLAMPED_SWIGLU) {
@@ -985,7 +1059,7 @@ template <int KIND, int DP>
 __global__ void __launch_bounds__(64) sv_lin_scan_kernel(const KrSvLin a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int TB = 8;
-    constexpr bool ML = KIND == 3;
+    constexpr bool ML = KIND == 3, GLA = KIND == 4, SSD = KIND == 5;
     const int e = blockIdx.x, h = blockIdx.y, cb = blockIdx.z, lane = threadIdx.x;
     const int part = lane & 3, cl = lane >> 2, col = cb * 16 + cl;
     const int dim = a.dim, vdim = a.vdim, H = a.heads, ncb = (vdim + 15) / 16;
@@ -1003,11 +1077,37 @@ __global__ void __launch_bounds__(64) sv_lin_scan_kernel(const KrSvLin a) {
         n[r] = (ML && ok) ? nmg[row] : 0.0f;
     }
     float m = (ML && !fresh) ? nmg[dim] : 0.0f;
-    const float decay = ML ? 0.0f : a.decay[h];
-    float* qs = lds; float* ks = qs + TB * dimp; float* vs = ks + TB * dimp; float* gs = vs + TB * 16;
+    const float decay = KIND == 2 ? a.decay[h] : 0.0f;
+    float* qs = lds; float* ks = qs + TB * dimp; float* vs = ks + TB * dimp; float* gs = vs + TB * 16; float* as = gs + TB * 2;      // as [TB * dimp]: per-channel decays (gla)
     const int half = a.rot_dims / 2;
     for (int tb = t0; tb < t1; tb += TB) {
         const int nt = min(TB, t1 - tb);
+        if constexpr (GLA || SSD) {
+            const int hq = h / a.qk_group;
+            for (int idx = lane; idx < nt * dimp; idx += 64) {
+                const int tt = idx / dimp, d = idx - tt * dimp;
+                const size_t r = (size_t)(tb + tt) * a.src_ld + (size_t)hq * dim + d;
+                qs[idx] = d < dim ? a.qsrc[r] * a.q_scale : 0.0f;
+                ks[idx] = d < dim ? a.ksrc[r] * a.k_scale : 0.0f;
+                if constexpr (GLA) {
+                    float al = 0.0f;
+                    if (d < dim) {
+                        const float z = a.gz[(size_t)(tb + tt) * a.gz_ld + (size_t)h * dim + d] + a.gz_bias[(size_t)h * dim + d];
+                        al = expf((fminf(z, 0.0f) - log1pf(expf(-fabsf(z)))) * a.inv_tau);      // sigmoid(z)^(1 / tau)
+                    }
+                    as[idx] = al;
+                }
+            }
+            for (int idx = lane; idx < nt * 16; idx += 64) {
+                const int tt = idx >> 4, c = cb * 16 + (idx & 15);
+                vs[idx] = c < vdim ? a.vsrc[(size_t)(tb + tt) * a.src_ld + (size_t)h * vdim + c] : 0.0f;
+            }
+            if (SSD && lane < nt) {
+                const float z = a.dtz[(size_t)(tb + lane) * a.dtz_ld + h] + a.dt_bias[h];
+                const float dt = fmaxf(z, 0.0f) + log1pf(expf(-fabsf(z)));                      // softplus
+                gs[2 * lane] = dt; gs[2 * lane + 1] = -expf(a.a_log[h]) * dt;
+            }
+        } else {
         for (int idx = lane; idx < nt * dimp; idx += 64) {
             const int tt = idx / dimp, d = idx - tt * dimp;
             const float* zr = a.z + (size_t)(tb + tt) * a.ld + (size_t)h * dim;
@@ -1024,6 +1124,7 @@ __global__ void __launch_bounds__(64) sv_lin_scan_kernel(const KrSvLin a) {
             if (a.gate_cap > 0.0f) { zi = a.gate_cap * tanhf(zi / a.gate_cap); zf = a.gate_cap * tanhf(zf / a.gate_cap); }
             gs[2 * lane] = zi;
             gs[2 * lane + 1] = fminf(zf, 0.0f) - log1pf(expf(-fabsf(zf)));      // log sigmoid
+        }
         }
         SV_WAVE_SYNC();
         if (half > 0) {
@@ -1045,14 +1146,17 @@ __global__ void __launch_bounds__(64) sv_lin_scan_kernel(const KrSvLin a) {
                 const float ig = gs[2 * tt], fg = gs[2 * tt + 1];
                 const float mn = fmaxf(fg + m, ig);
                 av = expf(fg + m - mn); bv = expf(ig - mn); m = mn;
-            } else { av = decay; bv = 1.0f; }
+            } else if constexpr (SSD) { bv = gs[2 * tt]; av = expf(gs[2 * tt + 1]); }
+            else { av = decay; bv = 1.0f; }
+            const float* ap = as + tt * dimp + part * dpr;
             const float bvv = bv * v;
             float po = 0.0f, pn = 0.0f;
 #pragma unroll
             for (int r = 0; r < DP; r++) {
                 if (r < dpr) {
                     const float kr = kp[r], qr = qp[r];
-                    S[r] = __builtin_fmaf(kr, bvv, av * S[r]);
+                    if constexpr (GLA) S[r] = __builtin_fmaf(kr, bvv, ap[r] * S[r]);
+                    else S[r] = __builtin_fmaf(kr, bvv, av * S[r]);
                     po = __builtin_fmaf(S[r], qr, po);
                     if constexpr (ML) { n[r] = __builtin_fmaf(bv, kr, av * n[r]); pn = __builtin_fmaf(n[r], qr, pn); }
                 }
@@ -1372,9 +1476,27 @@ __global__ void __launch_bounds__(64) sv_lin_out_kernel(const KrSvLin a, T* __re
     for (int d = lane; d < vdim; d += 64) {
         const float gz = g[d], sg = 1.0f / (1.0f + expf(-gz));
         float v = o[d] * inv;
-        if (a.norm_w) v *= a.norm_w[(size_t)h * vdim + d];
+        if (a.norm_w) v *= a.norm_w[a.norm_shared ? (size_t)d : (size_t)h * vdim + d];
         sv_st(out + ((size_t)t * H + h) * vdim + d, v * (a.kind == 3 ? sg : gz * sg));
     }
+}
+
+// the selective state-space mixer after its scan (KrSvSsdOut): one workgroup per token, the gated row in LDS
+template <typename T>
+__global__ void __launch_bounds__(256) sv_ssd_out_kernel(const KrSvSsdOut a, T* __restrict__ out) {
+    extern __shared__ float yr[];            // [inner] | [2 * groups]
+    const size_t t = blockIdx.x;
+    const int inner = a.heads * a.vdim;
+    float* gst = yr + inner;
+    for (int c = threadIdx.x; c < inner; c += 256) {
+        const float xv = a.x[t * a.ld_x + c], zv = a.z[t * a.ld_z + c];
+        yr[c] = __builtin_fmaf(a.D[c / a.vdim], xv, a.o[t * inner + c]) * (zv / (1.0f + expf(-zv)));
+    }
+    __syncthreads();
+    sv_group_stats<KR_SV_NORM_RMS, 4>(yr, inner, a.groups, a.eps, gst);
+    __syncthreads();
+    const int gw = inner / a.groups;
+    for (int c = threadIdx.x; c < inner; c += 256) sv_st(out + t * a.out_ld + c, yr[c] * gst[2 * (c / gw) + 1] * a.w[c] * a.scale);
 }
 
 __global__ void __launch_bounds__(1024) sv_argmax_kernel(const float* __restrict__ logits, int vocab, int* __restrict__ out) {
@@ -1413,10 +1535,39 @@ void kr_sv_fill_uniform(void* p, bool f32, size_t n, uint64_t seed, float amp, h
     else hipLaunchKernelGGL(sv_fill_uniform_kernel<uint16_t>, grid, dim3(256), 0, st, (uint16_t*)p, n, seed, amp);
 }
 
-void kr_sv_embed(const void* table, bool f32, const int* tokens, float* x, void* h_out, int T, int width, float scale, hipStream_t st) {
+void kr_sv_embed(const void* table, bool f32, const int* tokens, float* x, void* h_out, int T, int width, float scale, const void* table2, const int* rows2, hipStream_t st) {
     if (T <= 0) return;
-    if (f32) hipLaunchKernelGGL(sv_embed_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)table, tokens, x, (float*)h_out, width, scale);
-    else hipLaunchKernelGGL(sv_embed_kernel<uint16_t>, dim3(T), dim3(256), 0, st, (const uint16_t*)table, tokens, x, (uint16_t*)h_out, width, scale);
+    if (f32) hipLaunchKernelGGL(sv_embed_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)table, tokens, x, (float*)h_out, width, scale, (const float*)table2, rows2);
+    else hipLaunchKernelGGL(sv_embed_kernel<uint16_t>, dim3(T), dim3(256), 0, st, (const uint16_t*)table, tokens, x, (uint16_t*)h_out, width, scale, (const uint16_t*)table2, rows2);
+}
+
+void kr_sv_stream_norm(float* x, const float* add, const float* w, const float* b, bool in_place, void* out, bool out_f32, int T, int width, float eps, int kind, int groups,
+                       hipStream_t st) {
+    if (T <= 0 || (!add && !w)) return;
+    const size_t lds = (size_t)(width + 2 * (groups > 1 ? groups : 0)) * sizeof(float);
+#define SV_SN(T_, K_) hipLaunchKernelGGL((sv_stream_norm_kernel<T_, K_>), dim3(T), dim3(256), lds, st, x, add, w, b, (int)in_place, (T_*)out, width, eps, groups)
+    if (kind == KR_SV_NORM_LAYER) { if (out_f32) SV_SN(float, KR_SV_NORM_LAYER); else SV_SN(uint16_t, KR_SV_NORM_LAYER); }
+    else { if (out_f32) SV_SN(float, KR_SV_NORM_RMS); else SV_SN(uint16_t, KR_SV_NORM_RMS); }
+#undef SV_SN
+}
+
+void kr_sv_chan_conv(const KrSvChanConv& c, hipStream_t st) {
+    if (c.T <= 0 || c.C <= 0) return;
+    hipLaunchKernelGGL(sv_chan_conv_kernel, dim3(c.T, (c.C + 255) / 256), dim3(256), 0, st, c);
+}
+void kr_sv_chan_conv_save(const KrSvChanConv& c, hipStream_t st) {
+    if (c.T <= 0 || c.C <= 0 || c.taps < 2 || c.n_entries <= 0) return;
+    hipLaunchKernelGGL(sv_chan_conv_save_kernel, dim3(c.n_entries, c.taps - 1, (c.C + 255) / 256), dim3(256), 0, st, c);
+}
+void kr_sv_scale(float* p, size_t n, float scale, hipStream_t st) {
+    if (n == 0) return;
+    hipLaunchKernelGGL(sv_scale_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p, n, scale);
+}
+void kr_sv_ssd_out(const KrSvSsdOut& a, bool f32, hipStream_t st) {
+    if (a.T <= 0) return;
+    const size_t lds = (size_t)(a.heads * a.vdim + 2 * a.groups) * sizeof(float);
+    if (f32) hipLaunchKernelGGL(sv_ssd_out_kernel<float>, dim3(a.T), dim3(256), lds, st, a, (float*)a.out);
+    else hipLaunchKernelGGL(sv_ssd_out_kernel<uint16_t>, dim3(a.T), dim3(256), lds, st, a, (uint16_t*)a.out);
 }
 
 void kr_sv_norm(const float* x, const int* rows, const float* w, const float* b, void* out, bool out_f32, int R, int width, float eps, int kind, int groups, float* out32,
@@ -1612,10 +1763,10 @@ void kr_sv_lin_scan(const KrSvLin& a, hipStream_t st) {
     if (a.T <= 0 || a.n_entries <= 0) return;
     const int dpr = (a.dim + 3) / 4;
     const dim3 grid(a.n_entries, a.heads, (a.vdim + 15) / 16);
-    const size_t lds = (size_t)(2 * 8 * 4 * dpr + 8 * 16 + 8 * 2) * sizeof(float);
+    const size_t lds = (size_t)((a.kind == 4 ? 3 : 2) * 8 * 4 * dpr + 8 * 16 + 8 * 2) * sizeof(float);
 #define SV_LIN(K_, DP_) hipLaunchKernelGGL((sv_lin_scan_kernel<K_, DP_>), grid, dim3(64), lds, st, a)
 #define SV_LIN_D(K_) do { if (dpr <= 8) SV_LIN(K_, 8); else if (dpr <= 16) SV_LIN(K_, 16); else if (dpr <= 32) SV_LIN(K_, 32); else if (dpr <= 64) SV_LIN(K_, 64); else SV_LIN(K_, 128); } while (0)
-    if (a.kind == 3) SV_LIN_D(3); else SV_LIN_D(2);
+    if (a.kind == 3) SV_LIN_D(3); else if (a.kind == 4) SV_LIN_D(4); else if (a.kind == 5) SV_LIN_D(5); else SV_LIN_D(2);
 #undef SV_LIN_D
 #undef SV_LIN
 }

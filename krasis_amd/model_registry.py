@@ -86,6 +86,12 @@ class ServeModelSpec:
     canon_taps: int = 0                  # > 1: the mixers read h + a causal convolution of h over the request's positions
     res_gate: int = 0                    # 1: sublayer outputs are gated by sigmoid(W h + b) before they join the stream
     extra: Optional[dict] = None         # per-layer arrays the design's config carries instead of the checkpoint (tensor name -> float32 array)
+    norm_weight_offset: float = 0.0      # 1: norm weights are stored around zero
+    embed_norm: int = 0                  # the embedding row is normed before the first layer
+    bigram: Optional[Tuple[int, int, int]] = None      # (buckets, multiplier of the previous token, multiplier of the token): a hashed pair embedding joins the row
+    logit_scale: float = 0.0             # 0: the logits as they are
+    row_of: Optional[Dict[str, int]] = None            # a design's own bookkeeping: which config layer / which pass a layer run stands for
+    fit: Optional[Callable[["ServeModelSpec", Callable[[str], Tuple[int, ...]]], None]] = None      # completes sizes that only tensor shapes give (called with name -> shape before the store is made)
 
 
 _ARCHITECTURES: Dict[str, Callable[[dict], ServeModelSpec]] = {}
@@ -336,6 +342,132 @@ def midisun_spec(cfg: dict) -> ServeModelSpec:
 register_architecture("Midisun", midisun_spec)
 
 
+# ---- Lufozen: pre-normed sequential layers with RMS norms whose weights are stored around zero.  The embedding row (scaled) plus a hashed pair-of-tokens row is
+# normed before the first layer.  A block of consecutive layers may run several times with the same tensors; every pass keeps its own cache and state, and a
+# vector of its own joins the stream right before it.  Three mixers.  'attention': biased projections, a short causal convolution on q, k, v, per-head weighted
+# q / k norm, interleaved partial rotation with banded frequency scaling, a zero-score sink in the softmax, an element-wise sigmoid gate on the output.
+# 'parallel': an un-biased attention (half-split rotation, plain softmax) and a state-space mixer side by side on the same input, their outputs weighted.
+# 'gla': linear attention whose state decays per key channel by a low-rank function of the input.  Feed-forward: un-gated, squared relu.  Logits scaled.
+def _lufozen_runs(cfg: dict) -> List[Tuple[int, Optional[int]]]:
+    """(layer of config.json, pass number if the run opens a pass of the repeated block) for every layer run, in order"""
+    n = len(cfg["layers"])
+    lp = cfg.get("loop")
+    if not lp:
+        return [(i, None) for i in range(n)]
+    a, b, times = int(lp["start"]), int(lp["stop"]), int(lp["times"])
+    if not 0 <= a <= b <= n or times < 1:
+        raise ValueError(f"loop {lp!r} over {n} layers")
+    runs: List[Tuple[int, Optional[int]]] = [(i, None) for i in range(a)]
+    for t in range(times):
+        runs += [(i, t if i == a else None) for i in range(a, b)]
+    return runs + [(i, None) for i in range(b, n)]
+
+
+def _lufozen_rot(l: S.LayerSpec, rot: Optional[dict], interleaved: int) -> None:
+    if not rot or not int(rot.get("dims", 0)):
+        return
+    l.rot_dims, l.rot_interleaved, l.rot_base = int(rot["dims"]), interleaved, float(rot["base"])
+    sc = rot.get("scaling")
+    if sc:
+        l.rot_scaling, l.rot_factor = S.ROT_BANDS, float(sc["factor"])
+        l.rot_original, l.rot_fast, l.rot_slow = float(sc["original"]), float(sc["high"]), float(sc["low"])
+
+
+def _lufozen_tensors(spec: ServeModelSpec) -> Iterator[Tuple[int, str, int, str]]:
+    yield -1, "embed", 0, "embed"
+    if spec.bigram:
+        yield -1, "bigram", 0, "bigram"
+    yield -1, "embed_norm", 0, "embed.norm"
+    yield -1, "final_norm_w", 0, "final.norm"
+    yield -1, "head", 0, "head"
+    for r, l in enumerate(spec.layers):
+        if l.pre_add:
+            yield r, "pre_add", 0, f"loop.step@{spec.row_of[f'run{r}']}"
+        if l.weights_of:
+            continue
+        p = f"l{spec.row_of[f'layer{r}']}"
+        yield r, "norm_w", 0, f"{p}.norm1"
+        if l.mixer_kind == S.MIX_GLA:
+            for role, n in (("q", "q"), ("k", "k"), ("v", "v"), ("out_gate", "g"), ("o", "o"), ("lin_norm", "norm"), ("decay_a1", "a1"), ("decay_a2", "a2"), ("decay_a2_b", "a2.b")):
+                yield r, role, 0, f"{p}.mix.{n}"
+        elif l.side_mixer == S.MIX_SSD:
+            for role, n in (("q", "q"), ("k", "k"), ("v", "v"), ("q_norm", "q.norm"), ("k_norm", "k.norm"), ("o", "o")):
+                yield r, role, 0, f"{p}.mix.left.{n}"
+            for role, n in (("ssd_in", "in"), ("ssd_conv", "conv"), ("ssd_conv_b", "conv.b"), ("ssd_dt_bias", "dt_bias"), ("ssd_a_log", "A_log"), ("ssd_d", "D"), ("ssd_norm", "norm"),
+                            ("ssd_o", "o")):
+                yield r, role, 0, f"{p}.mix.right.{n}"
+        else:
+            for role, n in (("q", "q"), ("k", "k"), ("v", "v"), ("q_bias", "q.b"), ("k_bias", "k.b"), ("v_bias", "v.b"), ("o_bias", "o.b"), ("q_norm", "q.norm"), ("k_norm", "k.norm"),
+                            ("out_gate", "g"), ("o", "o")):
+                yield r, role, 0, f"{p}.mix.{n}"
+            if l.proj_conv:
+                for role, n in (("q_conv", "q.conv"), ("k_conv", "k.conv"), ("v_conv", "v.conv")):
+                    yield r, role, 0, f"{p}.mix.{n}"
+        if l.mlp_kind == S.MLP_DENSE:
+            yield r, "norm2_w", 0, f"{p}.norm2"
+            yield r, "up", 0, f"{p}.mlp.up"
+            yield r, "down", 0, f"{p}.mlp.down"
+
+
+def lufozen_spec(cfg: dict) -> ServeModelSpec:
+    layers: List[S.LayerSpec] = []
+    row_of: Dict[str, int] = {}
+    first_run: Dict[int, int] = {}
+    for r, (i, opens) in enumerate(_lufozen_runs(cfg)):
+        lc = cfg["layers"][i]
+        kind, m = lc.get("type"), lc["mixer"]
+        if kind == "attention":
+            l = S.LayerSpec(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
+                            qk_unit_norm=S.QKNORM_WEIGHTED, scale=float(m["scale"]), has_sink=S.SINK_ZERO, proj_bias=2, proj_conv=int(m.get("conv") or 0),
+                            out_gate=S.OGATE_ELEM_SIGMOID)
+            _lufozen_rot(l, m.get("rot"), 1)
+        elif kind == "parallel":
+            a, b = m["left"], m["right"]
+            l = S.LayerSpec(heads=int(a["heads"]), kv_heads=int(a.get("kv_heads", a["heads"])), dim=int(a["dim"]), vdim=int(a.get("vdim", a["dim"])),
+                            qk_unit_norm=S.QKNORM_WEIGHTED, scale=float(a["scale"]), side_mixer=S.MIX_SSD, ssd_heads=int(b["heads"]), ssd_vdim=int(b["vdim"]),
+                            ssd_state=int(b["state"]), ssd_groups=int(b.get("groups", 1)), ssd_conv=int(b.get("conv") or 1), ssd_norm_groups=int(b.get("norm_groups", 1)),
+                            mix_scale=float(m.get("left_scale", 1.0)), side_scale=float(m.get("right_scale", 1.0)))
+            if l.mix_scale == 0.0 or l.side_scale == 0.0:
+                raise ValueError(f"layer {i}: a mixer weighted by zero")
+            _lufozen_rot(l, a.get("rot"), 0)
+        elif kind == "gla":
+            # the rank of the decay's projection pair is the checkpoint's (a1: [rank, width]) unless config.json names it: lufozen_fit_checkpoint
+            l = S.LayerSpec(heads=int(m["heads"]), kv_heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]), mixer_kind=S.MIX_GLA, lin_norm_weight=2,
+                            decay_rank=int(m.get("rank") or 0), decay_tau=float(m["tau"]))
+        else:
+            raise ValueError(f"layer {i}: mixer type {kind!r} is not part of this design")
+        mlp = lc.get("mlp")
+        if mlp is not None:
+            if mlp.get("kind") != "dense":
+                raise ValueError(f"layer {i}: feed-forward kind {mlp.get('kind')!r}")
+            l.mlp_kind, l.ff, l.dense_act = S.MLP_DENSE, int(mlp["ff"]), S.ACT_RELU2
+        if i in first_run:
+            l.weights_of = first_run[i] + 1
+        else:
+            first_run[i] = r
+        if opens is not None:
+            l.pre_add = 1
+            row_of[f"run{r}"] = opens
+        row_of[f"layer{r}"] = i
+        layers.append(l)
+    emb = cfg.get("embedding") or {}
+    bg = emb.get("bigram")
+    return ServeModelSpec(vocab=int(cfg["vocab"]), width=int(cfg["width"]), norm_kind=S.NORM_RMS, norm_eps=float(cfg["norm"]["eps"]), layers=layers,
+                          tensors=_lufozen_tensors, block_kind=S.BLOCK_SEQUENTIAL, pre_norm=1, post_norm=0, norm_bias=0, embed_scale=float(emb.get("scale", 1.0)),
+                          norm_weight_offset=1.0, embed_norm=1, bigram=(int(bg["buckets"]), int(bg["mul_prev"]), int(bg["mul_cur"])) if bg else None,
+                          logit_scale=float(cfg.get("logit_scale", 1.0)), row_of=row_of, fit=lufozen_fit_checkpoint)
+
+
+def lufozen_fit_checkpoint(spec: ServeModelSpec, shape_of: Callable[[str], Tuple[int, ...]]) -> None:
+    """sizes that only the checkpoint gives: the rank of a gla layer's decay projections"""
+    for r, l in enumerate(spec.layers):
+        if l.mixer_kind == S.MIX_GLA and not l.decay_rank:
+            l.decay_rank = int(shape_of(f"l{spec.row_of[f'layer{r}']}.mix.a1")[0])
+
+
+register_architecture("Lufozen", lufozen_spec)
+
+
 def read_config(model_dir: str) -> dict:
     with open(os.path.join(model_dir, "config.json")) as f:
         return json.load(f)
@@ -358,6 +490,8 @@ def load_model(model_dir: str, dtype: str = "bfloat16", max_tokens: int = 4096, 
     if fam.startswith("serve:"):
         from .scheduler import BatchEngine
         spec = _ARCHITECTURES[fam[6:]](cfg)
+        if spec.fit is not None:
+            spec.fit(spec, SafetensorsFile(os.path.join(model_dir, "model.safetensors")).shape)
         eng = BatchEngine(spec, dtype=dtype, max_tokens=max_tokens, max_slots=max_slots, device=device, build=build)
         eng.load_safetensors(os.path.join(model_dir, "model.safetensors"))
         return eng

@@ -17,6 +17,14 @@ from . import serve_store as S
 _DTYPES = {"bfloat16": S.BF16, "bf16": S.BF16, "float32": S.F32, "f32": S.F32}
 
 
+def _named(get, name: str):
+    """a checkpoint tensor, or with `tensor@row` one row of it (a table that holds one vector per pass of a repeated block)"""
+    if "@" in name:
+        base, row = name.rsplit("@", 1)
+        return get(base)[int(row)]
+    return get(name)
+
+
 class BatchEngine:
     def __init__(self, spec, dtype: str = "bfloat16", max_tokens: int = 4096, max_slots: int = 4, device: int = 0, build: bool = False):
         if dtype not in _DTYPES:
@@ -25,7 +33,8 @@ class BatchEngine:
         self.store = S.ServeStore(spec.vocab, spec.width, spec.layers, dtype=_DTYPES[dtype], norm_kind=spec.norm_kind, norm_eps=spec.norm_eps,
                                   max_slots=max_slots, pool_tokens=max_tokens, device=device, build=build, block_kind=spec.block_kind, pre_norm=spec.pre_norm,
                                   post_norm=spec.post_norm, norm_bias=spec.norm_bias, residual_mult=spec.residual_mult, norm_groups=spec.norm_groups,
-                                  embed_scale=spec.embed_scale, canon_taps=spec.canon_taps, res_gate=spec.res_gate)
+                                  embed_scale=spec.embed_scale, canon_taps=spec.canon_taps, res_gate=spec.res_gate, norm_weight_offset=spec.norm_weight_offset,
+                                  embed_norm=spec.embed_norm, bigram=spec.bigram, logit_scale=spec.logit_scale)
         self.vocab = spec.vocab
         self._slot: Dict[object, int] = {}
 
@@ -35,14 +44,14 @@ class BatchEngine:
         f = SafetensorsFile(path)
         extra = getattr(self.spec, "extra", None) or {}
         for layer, role, index, name in self.spec.tensors(self.spec):
-            self.store.set_tensor(layer, role, extra[name] if name in extra else f.get(name), index)
+            self.store.set_tensor(layer, role, extra[name] if name in extra else _named(f.get, name), index)
         self.store.finalize()
 
     def load_arrays(self, arrays: Dict[str, np.ndarray]) -> None:
         """tensors by checkpoint name: float32, or uint16 bf16 bit patterns"""
         extra = getattr(self.spec, "extra", None) or {}
         for layer, role, index, name in self.spec.tensors(self.spec):
-            self.store.set_tensor(layer, role, extra[name] if name in extra else arrays[name], index)
+            self.store.set_tensor(layer, role, extra[name] if name in extra else _named(arrays.__getitem__, name), index)
         self.store.finalize()
 
     def load_synthetic(self, seed: int = 1, amp: float = 1.0) -> None:

@@ -15,16 +15,16 @@ from ._lib import ServeConfigC, ServeLayerC, check_serve, load_serve_library
 BF16, F32 = 0, 1
 NORM_LAYER, NORM_RMS = 0, 1
 MLP_NONE, MLP_DENSE, MLP_MOE = 0, 1, 2
-ACT_GELU_TANH, ACT_CLAMPED_SWIGLU, ACT_SILU = 0, 1, 2
+ACT_GELU_TANH, ACT_CLAMPED_SWIGLU, ACT_SILU, ACT_RELU2 = 0, 1, 2, 3
 BLOCK_PARALLEL, BLOCK_SEQUENTIAL = 0, 1
-MIX_ATTENTION, MIX_LATENT, MIX_RETENTION, MIX_MLSTM = 0, 1, 2, 3
+MIX_ATTENTION, MIX_LATENT, MIX_RETENTION, MIX_MLSTM, MIX_GLA, MIX_SSD = 0, 1, 2, 3, 4, 5
 QKNORM_NONE, QKNORM_AFTER_ROT, QKNORM_WEIGHTED, QKNORM_WHOLE = 0, 1, 2, 3
 RBIAS_NONE, RBIAS_LOGIT, RBIAS_CHOICE = 0, 1, 2
 RSCORE_SOFTMAX, RSCORE_SIGMOID = 0, 1
 GSCORE_MAX, GSCORE_TOP2 = 0, 1
-OGATE_NONE, OGATE_HEAD_SIGMOID = 0, 1
+OGATE_NONE, OGATE_HEAD_SIGMOID, OGATE_ELEM_SIGMOID = 0, 1, 2
 SINK_NONE, SINK_TENSOR, SINK_ZERO = 0, 1, 2
-ROT_LINEAR, ROT_BY_PARTS = 0, 1
+ROT_LINEAR, ROT_BY_PARTS, ROT_BANDS = 0, 1, 2
 VMIX_NONE, VMIX_FIRST, VMIX_BLEND = 0, 1, 2
 PAGE_TOKENS = 64
 ROLES = {n: i for i, n in enumerate(["embed", "final_norm_w", "final_norm_b", "head", "norm_w", "norm_b", "q", "k", "v", "o", "sink", "gate", "up", "down",
@@ -32,7 +32,9 @@ ROLES = {n: i for i, n in enumerate(["embed", "final_norm_w", "final_norm_b", "h
                                      "norm2_w", "norm2_b", "post1_w", "post1_b", "post2_w", "post2_b", "q_norm", "k_norm", "vmix", "router_bias",
                                      "dq", "dq_norm", "uq", "dkv", "dkv_norm", "uk", "uv",
                                      "q_bias", "k_bias", "o_bias", "out_gate", "canon", "res_gate1", "res_gate1_b", "res_gate2", "res_gate2_b",
-                                     "lin_norm", "lin_decay", "igate", "igate_b", "fgate", "fgate_b"])}
+                                     "lin_norm", "lin_decay", "igate", "igate_b", "fgate", "fgate_b",
+                                     "embed_norm", "bigram", "pre_add", "v_bias", "q_conv", "k_conv", "v_conv", "decay_a1", "decay_a2", "decay_a2_b",
+                                     "ssd_in", "ssd_conv", "ssd_conv_b", "ssd_dt_bias", "ssd_a_log", "ssd_d", "ssd_norm", "ssd_o"])}
 
 
 @dataclass
@@ -86,13 +88,28 @@ class LayerSpec:
     lin_norm_weight: int = 0
     router_score: int = RSCORE_SOFTMAX
     group_score: int = GSCORE_MAX
+    weights_of: int = 0                  # 1 + the earlier layer whose tensors this layer uses (a block of layers that runs again); 0: its own
+    pre_add: int = 0                     # tensor pre_add [width] joins the stream before the layer
+    proj_conv: int = 0                   # taps of the causal convolution on q, k, v
+    decay_rank: int = 0                  # gla: rank of the decay's projection pair, and the root taken of its sigmoid
+    decay_tau: float = 0.0
+    side_mixer: int = 0                  # MIX_SSD: a state-space mixer beside the attention mixer, on the same input
+    ssd_heads: int = 0
+    ssd_vdim: int = 0
+    ssd_state: int = 0
+    ssd_groups: int = 0
+    ssd_conv: int = 0
+    ssd_norm_groups: int = 0
+    mix_scale: float = 0.0               # weights of the two mixers' outputs (0 reads as 1)
+    side_scale: float = 0.0
 
 
 class ServeStore:
     def __init__(self, vocab: int, width: int, layers: Sequence[LayerSpec], dtype: int = BF16, norm_kind: int = NORM_LAYER, norm_eps: float = 1e-5,
                  max_slots: int = 4, pool_tokens: int = 4096, page_tokens: int = PAGE_TOKENS, device: int = 0, build: bool = False,
                  block_kind: int = BLOCK_PARALLEL, pre_norm: int = 1, post_norm: int = 0, norm_bias: Optional[int] = None, residual_mult: float = 1.0,
-                 norm_groups: int = 0, embed_scale: float = 0.0, canon_taps: int = 0, res_gate: int = 0):
+                 norm_groups: int = 0, embed_scale: float = 0.0, canon_taps: int = 0, res_gate: int = 0, norm_weight_offset: float = 0.0, embed_norm: int = 0,
+                 bigram: Optional[Tuple[int, int, int]] = None, logit_scale: float = 0.0):
         self._lib = load_serve_library(build=build)
         self.vocab, self.width, self.layers, self.dtype = vocab, width, list(layers), dtype
         self.page_tokens = page_tokens
@@ -101,7 +118,7 @@ class ServeStore:
         if norm_bias is None:
             norm_bias = int(norm_kind == NORM_LAYER)
         cfg = ServeConfigC(vocab, width, len(self.layers), dtype, norm_kind, norm_eps, max_slots, page_tokens, pool_tokens, block_kind, pre_norm, post_norm, norm_bias,
-                           residual_mult, norm_groups, embed_scale, canon_taps, res_gate)
+                           residual_mult, norm_groups, embed_scale, canon_taps, res_gate, norm_weight_offset, embed_norm, *(bigram or (0, 0, 0)), logit_scale)
         arr = (ServeLayerC * len(self.layers))()
         for i, l in enumerate(self.layers):
             for f in fields(LayerSpec):
