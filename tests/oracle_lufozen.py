@@ -4,7 +4,10 @@ No cache, no state object, no code shared with the package: the recurrences are 
 positions, attention as a full score matrix.  `forward(cfg, w, tokens)` returns the logits of every position and the residual stream after every
 layer run.  `w` maps checkpoint tensor names to float arrays; `cfg` is the dictionary of config.json.
 """
+import json
 import math
+import os
+import struct
 
 import numpy as np
 
@@ -16,10 +19,6 @@ def rms_unit(x, eps):
 def norm_one_plus(x, w, eps):
     """weight stored around zero"""
     return rms_unit(x, eps) * (1.0 + w)
-
-
-def gelu_tanh(z):
-    return 0.5 * z * (1.0 + np.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
 
 
 def silu(z):
@@ -220,6 +219,7 @@ def layer_order(cfg):
 
 
 def forward(cfg, w, tokens):
+    w = {k: np.asarray(v, np.float64) for k, v in w.items()}
     eps = float(cfg["norm"]["eps"])
     x = embed(cfg, w, tokens)
     streams = []
@@ -233,3 +233,130 @@ def forward(cfg, w, tokens):
         streams.append(x.copy())
     logits = norm_one_plus(x, w["final.norm"], eps) @ w["head"].T * float(cfg.get("logit_scale", 1.0))
     return logits, np.stack(streams)
+
+
+# ------------------------------------------------------------------------------------------------------------------------------------
+# small configurations and random weights for the tests
+# ------------------------------------------------------------------------------------------------------------------------------------
+def rot(dims, base=10000.0, factor=None, low=1.0, high=4.0, original=64):
+    r = {"dims": dims, "base": base}
+    if factor is not None:
+        r["scaling"] = {"factor": factor, "low": low, "high": high, "original": original}
+    return r
+
+
+def attn(heads, kv_heads, dim, vdim, scale=0.3, conv=3, rot=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "conv": conv}
+    if rot:
+        m["rot"] = rot
+    return "attention", m
+
+
+def left(heads, kv_heads, dim, vdim, scale=0.3, rot=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale}
+    if rot:
+        m["rot"] = rot
+    return m
+
+
+def ssd(heads, vdim, state, groups=1, conv=4, norm_groups=1):
+    return {"heads": heads, "vdim": vdim, "state": state, "groups": groups, "conv": conv, "norm_groups": norm_groups}
+
+
+def parallel(a, b, left_scale=0.7, right_scale=0.4):
+    return "parallel", {"left": a, "right": b, "left_scale": left_scale, "right_scale": right_scale}
+
+
+def gla(heads, dim, vdim, tau=8.0):
+    return "gla", {"heads": heads, "dim": dim, "vdim": vdim, "tau": tau}
+
+
+def dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def layer(mixer, mlp):
+    return {"type": mixer[0], "mixer": mixer[1], "mlp": mlp}
+
+
+def make_config(width, vocab, layers, eps=1e-5, embed_scale=3.0, bigram=(53, 7, 11), loop=None, logit_scale=0.7):
+    cfg = {"architecture": "Lufozen", "vocab": vocab, "width": width, "norm": {"eps": eps}, "layers": layers, "logit_scale": logit_scale,
+           "embedding": {"scale": embed_scale, "bigram": {"buckets": bigram[0], "mul_prev": bigram[1], "mul_cur": bigram[2]}}}
+    if loop:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return cfg
+
+
+def random_weights(cfg, seed, rank=6):
+    rng = np.random.default_rng(seed)
+    W, V = cfg["width"], cfg["vocab"]
+    out = {}
+
+    def mat(name, o, i, gain=1.0):
+        out[name] = (rng.standard_normal((o, i)) * gain / math.sqrt(i)).astype(np.float32)
+
+    def vec(name, n, mid=0.0, amp=0.1):
+        out[name] = (mid + amp * rng.standard_normal(n)).astype(np.float32)
+    out["embed"] = (rng.standard_normal((V, W)) * 0.5).astype(np.float32)
+    out["bigram"] = (rng.standard_normal((cfg["embedding"]["bigram"]["buckets"] + 1, W)) * 0.8).astype(np.float32)
+    vec("embed.norm", W); vec("final.norm", W)
+    mat("head", V, W)
+    times = int(cfg["loop"]["times"]) if cfg.get("loop") else 1
+    out["loop.step"] = (0.4 * rng.standard_normal((times, W))).astype(np.float32)
+    for i, lc in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", lc["mixer"]
+        vec(p + "norm1", W)
+        if lc["type"] == "attention":
+            H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            mat(p + "mix.q", H * d, W); mat(p + "mix.k", G * d, W); mat(p + "mix.v", G * dv, W); mat(p + "mix.g", H * dv, W); mat(p + "mix.o", W, H * dv)
+            vec(p + "mix.q.b", H * d, amp=0.3); vec(p + "mix.k.b", G * d, amp=0.3); vec(p + "mix.v.b", G * dv, amp=0.3); vec(p + "mix.o.b", W, amp=0.3)
+            vec(p + "mix.q.norm", d, 1.0, 0.2); vec(p + "mix.k.norm", d, 1.0, 0.2)
+            if m.get("conv"):
+                for n, c in (("q", H * d), ("k", G * d), ("v", G * dv)):
+                    out[p + f"mix.{n}.conv"] = (rng.standard_normal((c, m["conv"])) * 0.6).astype(np.float32)
+        elif lc["type"] == "parallel":
+            a, b = m["left"], m["right"]
+            H, G, d, dv = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+            q = p + "mix.left."
+            mat(q + "q", H * d, W); mat(q + "k", G * d, W); mat(q + "v", G * dv, W); mat(q + "o", W, H * dv)
+            vec(q + "q.norm", d, 1.0, 0.2); vec(q + "k.norm", d, 1.0, 0.2)
+            nh, sv, N, sg = b["heads"], b["vdim"], b["state"], b["groups"]
+            inner, cc = nh * sv, nh * sv + 2 * sg * N
+            q = p + "mix.right."
+            mat(q + "in", 2 * inner + 2 * sg * N + nh, W); mat(q + "o", W, inner)
+            out[q + "conv"] = (rng.standard_normal((cc, b["conv"])) * 0.6).astype(np.float32)
+            vec(q + "conv.b", cc, amp=0.2); vec(q + "dt_bias", nh, -0.5, 1.0); vec(q + "A_log", nh, -0.5, 1.0); vec(q + "D", nh, 1.0, 0.3); vec(q + "norm", inner, 1.0, 0.2)
+        else:
+            H, d, dv = m["heads"], m["dim"], m["vdim"]
+            q = p + "mix."
+            mat(q + "q", H * d, W); mat(q + "k", H * d, W); mat(q + "v", H * dv, W); mat(q + "g", H * dv, W); mat(q + "o", W, H * dv)
+            mat(q + "a1", rank, W); mat(q + "a2", H * d, rank, 2.0); vec(q + "a2.b", H * d, 2.0, 1.5); vec(q + "norm", dv, 1.0, 0.2)
+        if lc.get("mlp"):
+            vec(p + "norm2", W)
+            mat(p + "mlp.up", lc["mlp"]["ff"], W); mat(p + "mlp.down", W, lc["mlp"]["ff"])
+    return out
+
+
+def bf16_round(a):
+    """float32 -> the nearest bfloat16 (ties to even), back as float32"""
+    b = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    b = ((b + 0x7FFF + ((b >> 16) & 1)) >> 16) << 16
+    return b.astype(np.uint32).view(np.float32).reshape(np.shape(a))
+
+
+def write_checkpoint(path, cfg, W):
+    """config.json + model.safetensors with the weights as bfloat16 (the caller's oracle should use bf16_round of W)"""
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    header, blobs, at = {}, [], 0
+    for name, a in W.items():
+        raw = (np.ascontiguousarray(bf16_round(a), np.float32).view(np.uint32) >> 16).astype("<u2").tobytes()
+        header[name] = {"dtype": "BF16", "shape": list(np.shape(a)), "data_offsets": [at, at + len(raw)]}
+        blobs.append(raw); at += len(raw)
+    hj = json.dumps(header).encode()
+    hj += b" " * (-len(hj) % 8)
+    with open(os.path.join(path, "model.safetensors"), "wb") as f:
+        f.write(struct.pack("<Q", len(hj))); f.write(hj)
+        for b in blobs:
+            f.write(b)
