@@ -347,9 +347,9 @@ def parse():
                          "sizes -- prompt pass and decode throughput, kernel-family times -- beside the closest model of the decode graph (GQA + softmax top-k MoE, INT4) at "
                          "the same sizes; prints its own JSON line")
     ap.add_argument("--arch-sizes", default="small,large", help="sizes of --arch-compare (ARCH_SIZES)")
-    ap.add_argument("--arch-design", default="lomutar", choices=["lomutar", "pamulix", "midisun"],
+    ap.add_argument("--arch-design", default="lomutar", choices=["lomutar", "pamulix", "midisun", "lufozen"],
                     help="which layer-described design --arch-compare measures: lomutar (beside the decode graph's GQA + MoE model), pamulix or midisun (beside "
-                         "Lomutar, both on the batched serving store, at the same layer sizes)")
+                         "Lomutar), lufozen (beside Midisun with a dense feed-forward) -- both on the batched serving store, at the same layer sizes")
     return ap.parse_args()
 
 
@@ -670,6 +670,116 @@ def arch_compare_midisun(args):
                                    "gemm_family_frac_of_hbm_peak": byts / (d["family_ms"][1] * 1e-3) / 1e9 / HBM_PEAK_GBS}
         res["lomutar"] = r
         del eng; gc.collect()
+        out["sizes"][name] = res
+    flush_native_stdout()
+    print(json.dumps(out), flush=True)
+    return out
+
+
+def lufozen_serve_engine(z, kinds, ff):
+    """A Lufozen model with random bf16 weights on the batched serving store at the layer sizes z (ARCH_SIZES); kinds: one letter per layer, A = attention
+    (biased projections, three-tap convolution on q / k / v, per-head norms, rotation on half of a head with banded scaling, zero-score sink, element-wise
+    gate), P = attention and a state-space mixer side by side (state-space heads: the size's head count, head size as channels, 128 states in 8 groups,
+    four taps), G = gla (the size's heads, keys and values of the head size, decay projections of rank 16).  Every layer: an un-gated squared-relu
+    feed-forward of ff columns.  The second and third layer form a block that runs twice."""
+    from krasis_amd import model_registry as R, scheduler as SCH, serve_store as S
+    W, H, G, D, V, P = (z[c] for c in ("width", "heads", "kv_heads", "dim", "vocab", "prompt"))
+    rot = dict(rot_dims=D // 2, rot_base=5e5, rot_scaling=S.ROT_BANDS, rot_factor=8.0, rot_original=8192.0, rot_fast=4.0, rot_slow=1.0)
+    mlp = dict(mlp_kind=S.MLP_DENSE, ff=ff, dense_act=S.ACT_RELU2)
+    mk = {"A": lambda: S.LayerSpec(heads=H, kv_heads=G, dim=D, vdim=D, qk_unit_norm=S.QKNORM_WEIGHTED, scale=D ** -0.5, has_sink=S.SINK_ZERO, proj_bias=2, proj_conv=3,
+                                   out_gate=S.OGATE_ELEM_SIGMOID, rot_interleaved=1, **rot, **mlp),
+          "P": lambda: S.LayerSpec(heads=H, kv_heads=G, dim=D, vdim=D, qk_unit_norm=S.QKNORM_WEIGHTED, scale=D ** -0.5, rot_interleaved=0, side_mixer=S.MIX_SSD, ssd_heads=H,
+                                   ssd_vdim=D, ssd_state=128, ssd_groups=min(8, H), ssd_conv=4, ssd_norm_groups=min(8, H), mix_scale=0.6, side_scale=0.5, **rot, **mlp),
+          "G": lambda: S.LayerSpec(heads=H, kv_heads=H, dim=D, vdim=D, mixer_kind=S.MIX_GLA, lin_norm_weight=2, decay_rank=16, decay_tau=16.0, **mlp)}
+    layers = [mk[c]() for c in kinds]
+    if len(layers) >= 3:          # layers 1 and 2 run twice: [0, 1, 2, 1', 2', 3 ...]
+        again = [mk[c]() for c in kinds[1:3]]
+        for j, l in enumerate(again):
+            l.weights_of = 2 + j
+        layers[1].pre_add = 1; again[0].pre_add = 1
+        layers = layers[:3] + again + layers[3:]
+    spec = R.ServeModelSpec(V, W, S.NORM_RMS, 1e-5, layers, None, block_kind=S.BLOCK_SEQUENTIAL, pre_norm=1, post_norm=0, norm_bias=0, embed_scale=16.0, norm_weight_offset=1.0,
+                            embed_norm=1, bigram=(4093, 31, 17), logit_scale=0.5)
+    eng = SCH.BatchEngine(spec, dtype="bfloat16", max_tokens=4 * (P + 256), max_slots=4)
+    eng.load_synthetic(seed=7, amp=1.0)
+    return eng, len(layers)
+
+
+def arch_compare_lufozen(args):
+    """The Lufozen design beside Midisun (the closest design on the store: sequential pre-normed RMS blocks, attention and recurrent mixers), both with random
+    bf16 weights and a dense feed-forward of top x expert-ff columns, at the layer sizes of ARCH_SIZES.  Four Lufozen models per size: the mixed order
+    attention, parallel, gla, attention with the middle block run twice (the throughput), and one mixer kind alone each (what its kernels reach).
+    Mixer flops are the design's own: 4 x keys x dim per query for attention, 4 (state space) or 5 (gla: one more product for the per-channel decay) per
+    state element and token for the recurrences."""
+    import numpy as np
+    from krasis_amd import model_registry as R, scheduler as SCH, serve_store as S
+    out = {"metric": "arch_compare_lufozen_vs_midisun", "unit": "tok/s", "sizes": {}}
+    for name in [x for x in args.arch_sizes.split(",") if x]:
+        z = ARCH_SIZES[name]; W, H, G, D, L, V, P = (z[c] for c in ("width", "heads", "kv_heads", "dim", "layers", "vocab", "prompt"))
+        ff = z["top"] * z["ff"]
+        res = {"shape": dict(z), "dense_ff": ff}
+        N, SG = 128, min(8, H)
+        w_ff = 2 * W * ff                                             # up and down
+        w_att = (2 * H * D + 2 * G * D) * W + W * H * D               # q, k, v, the element-wise gate, the output projection
+        w_par = (H * D + 2 * G * D) * W + (2 * H * D + 2 * SG * N + H) * W + W * 2 * H * D
+        w_gla = 4 * H * D * W + 16 * W + H * D * 16 + W * H * D
+        att_flops = 2.0 * 2 * H * D * sum(i + 1 for i in range(P))   # causal, no window
+        rec_flops = {"P": 4.0 * P * H * D * N, "G": 5.0 * P * H * D * D}
+        state = {"P": H * D * N, "G": H * D * D}
+        order = "".join("APGA"[i % 4] for i in range(L))
+        for label, kinds in (("mixed_" + order, order), ("attention_only", "A" * L), ("parallel_only", "P" * L), ("gla_only", "G" * L)):
+            eng, runs = lufozen_serve_engine(z, kinds, ff)
+            ran = kinds[:3] + kinds[1:3] + kinds[3:] if len(kinds) >= 3 else kinds
+            m = serve_measure(eng, V, P, np.random.default_rng(3), decode_batches=(1, 4) if label.startswith("mixed") else (1,))
+            nA, nP, nG = ran.count("A"), ran.count("P"), ran.count("G")
+            macs_tok = nA * w_att + nP * w_par + nG * w_gla + runs * w_ff
+            fam = m["prefill_family_ms"]
+            mix_flops = (nA + nP) * att_flops + nP * rec_flops["P"] + nG * rec_flops["G"]
+            r = {"layer_runs": runs, "prefill": {"tok_s": P / m["prefill_s"], "ms": m["prefill_s"] * 1e3, "tokens": P, "family_ms": {n: round(v, 3) for n, v in zip(SERVE_FAMILIES, fam)},
+                                                 "gemm_family_frac_of_bf16_peak": 2.0 * P * (macs_tok + V * W / P) / (fam[1] * 1e-3) / 1e12 / F16_PEAK_TFLOPS,
+                                                 "mixer_family_TFLOPs": mix_flops / (fam[3] * 1e-3) / 1e12}}
+            r["prefill"]["mixer_frac_of_f32_peak"] = r["prefill"]["mixer_family_TFLOPs"] / F32_MATRIX_PEAK_TFLOPS
+            for B, d in m["decode"].items():
+                st_b = 2.0 * 4 * B * (nP * state["P"] + nG * state["G"])          # the matrix states, read and written, f32
+                # weights are read once per step whatever the number of runs that share them would suggest: every run reads them again
+                byts = 2.0 * (nA * w_att + nP * w_par + nG * w_gla + runs * w_ff + V * W) + st_b
+                r["decode_b%d" % B] = {"tok_s": B / d["s_per_step"], "ms_per_step": d["s_per_step"] * 1e3, "weight_and_state_bytes_per_step": byts,
+                                       "frac_of_hbm_peak": byts / d["s_per_step"] / 1e9 / HBM_PEAK_GBS, "family_ms": {n: round(v, 4) for n, v in zip(SERVE_FAMILIES, d["family_ms"])},
+                                       "gemm_family_frac_of_hbm_peak": (byts - st_b) / (d["family_ms"][1] * 1e-3) / 1e9 / HBM_PEAK_GBS, "state_bytes_per_step": st_b}
+            res["lufozen_" + label] = r
+            del eng; gc.collect()
+        # ---------------- Midisun at the same sizes with the same dense feed-forward width (SiLU-gated: three matrices), as many layers as Lufozen has runs
+        runs = L + 2 if L >= 3 else L
+        mk = {"A": lambda: S.LayerSpec(heads=H, kv_heads=G, dim=D, vdim=D, qk_unit_norm=S.QKNORM_WHOLE, scale=D ** -0.5, window=z["window"], has_sink=S.SINK_TENSOR, dist_bias=1,
+                                       proj_bias=1, v_from_k=1, softcap=30.0, out_gate=S.OGATE_HEAD_SIGMOID, mlp_kind=S.MLP_DENSE, ff=ff, dense_act=S.ACT_SILU),
+              "R": lambda: S.LayerSpec(heads=H, kv_heads=H, dim=D, vdim=D, mixer_kind=S.MIX_RETENTION, rot_dims=D, rot_interleaved=0, rot_base=1e6, mlp_kind=S.MLP_DENSE, ff=ff,
+                                       dense_act=S.ACT_SILU),
+              "M": lambda: S.LayerSpec(heads=H, kv_heads=H, dim=D, vdim=D, mixer_kind=S.MIX_MLSTM, gate_cap=12.0, lin_norm_weight=1, mlp_kind=S.MLP_DENSE, ff=ff, dense_act=S.ACT_SILU)}
+        for label, kinds in (("mixed", "".join("ARMA"[i % 4] for i in range(runs))), ("attention_only", "A" * runs), ("retention_only", "R" * runs)):
+            spec = R.ServeModelSpec(V, W, S.NORM_RMS, 1e-5, [mk[c]() for c in kinds], None, block_kind=S.BLOCK_SEQUENTIAL, pre_norm=1, post_norm=0, norm_bias=0, norm_groups=4,
+                                    embed_scale=2.0, canon_taps=4, res_gate=1)
+            eng = SCH.BatchEngine(spec, dtype="bfloat16", max_tokens=4 * (P + 256), max_slots=4)
+            eng.load_synthetic(seed=7, amp=1.0)
+            m = serve_measure(eng, V, P, np.random.default_rng(3), decode_batches=(1, 4) if label == "mixed" else (1,))
+            nA, nR = kinds.count("A"), kinds.count("R") + kinds.count("M")
+            w_att_m = (H * D + G * D + H) * W + W * H * D
+            w_rec_m = 4 * H * D * W + W * H * D
+            macs_tok = nA * w_att_m + nR * w_rec_m + runs * (3 * W * ff + 2 * W * W)
+            att_w = 2.0 * 2 * H * D * sum(min(i + 1, z["window"]) for i in range(P))
+            fam = m["prefill_family_ms"]
+            mix_flops = nA * att_w + kinds.count("R") * 4.0 * P * H * D * D + kinds.count("M") * 6.0 * P * H * D * D
+            r = {"layers": runs, "prefill": {"tok_s": P / m["prefill_s"], "ms": m["prefill_s"] * 1e3, "tokens": P, "family_ms": {n: round(v, 3) for n, v in zip(SERVE_FAMILIES, fam)},
+                                             "gemm_family_frac_of_bf16_peak": 2.0 * P * (macs_tok + V * W / P) / (fam[1] * 1e-3) / 1e12 / F16_PEAK_TFLOPS,
+                                             "mixer_family_TFLOPs": mix_flops / (fam[3] * 1e-3) / 1e12}}
+            r["prefill"]["mixer_frac_of_f32_peak"] = r["prefill"]["mixer_family_TFLOPs"] / F32_MATRIX_PEAK_TFLOPS
+            for B, d in m["decode"].items():
+                st_b = 2.0 * 4 * B * nR * H * D * D
+                byts = 2.0 * (nA * w_att_m + nR * w_rec_m + runs * (3 * W * ff + 2 * W * W) + V * W) + st_b
+                r["decode_b%d" % B] = {"tok_s": B / d["s_per_step"], "ms_per_step": d["s_per_step"] * 1e3, "weight_and_state_bytes_per_step": byts,
+                                       "frac_of_hbm_peak": byts / d["s_per_step"] / 1e9 / HBM_PEAK_GBS, "family_ms": {n: round(v, 4) for n, v in zip(SERVE_FAMILIES, d["family_ms"])},
+                                       "gemm_family_frac_of_hbm_peak": (byts - st_b) / (d["family_ms"][1] * 1e-3) / 1e9 / HBM_PEAK_GBS, "state_bytes_per_step": st_b}
+            res["midisun_" + label] = r
+            del eng; gc.collect()
         out["sizes"][name] = res
     flush_native_stdout()
     print(json.dumps(out), flush=True)
@@ -1634,7 +1744,7 @@ def main_multi(args, torch, dist, world, rank, local_rank):
 def main():
     args = parse()
     if args.arch_compare:
-        return {"pamulix": arch_compare_pamulix, "midisun": arch_compare_midisun}.get(args.arch_design, arch_compare)(args)
+        return {"pamulix": arch_compare_pamulix, "midisun": arch_compare_midisun, "lufozen": arch_compare_lufozen}.get(args.arch_design, arch_compare)(args)
     import torch
     import torch.distributed as dist
 

@@ -998,7 +998,12 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
                 q.q_scale = isd; q.k_scale = 1.0f;
             }
             q.ent_chunk0 = d_echunk; q.n_chunks = n_chunks; q.tok = (float4*)s->lin_tok.p; q.sbuf = (float*)s->lin_sbuf.p; q.nbuf = (float*)s->lin_nbuf.p; q.cmeta = (float*)s->lin_cm.p;
-            { Timer tm(s, 3); if (lin_chunked && l.chunkable() && kr_sv_lin_chunked_fits(d.dim, d.vdim)) kr_sv_lin_chunked(q, st); else kr_sv_lin_scan(q, st); }
+            {
+                Timer tm(s, 3);
+                if (lin_chunked && l.chunkable() && kr_sv_lin_chunked_fits(d.dim, d.vdim)) kr_sv_lin_chunked(q, st);
+                else if (lin_chunked && kr_sv_lin_scan_wide_fits(q.kind, d.dim)) kr_sv_lin_scan_wide(q, st);
+                else kr_sv_lin_scan(q, st);
+            }
             { Timer tm(s, 2); kr_sv_lin_out(q, s->f32, st); }
         } else if (l.ssd_alone()) {
             // no first mixer: the state-space mixer below is the layer's only one
@@ -1066,7 +1071,7 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
             q.dtz = zin + inner + cc; q.dtz_ld = l.n_h; q.dt_bias = (const float*)l.dt_bias.p; q.a_log = (const float*)l.a_log.p;
             q.state = (float*)run.ssd_state.p; q.state_stride = l.ssd_state_stride;
             q.ent_off = d_eoff; q.ent_slot = d_eslot; q.n_entries = n_entries; q.pos = d_pos; q.T = T; q.o = (float*)s->lin_o.p;
-            { Timer tm(s, 3); kr_sv_lin_scan(q, st); }
+            { Timer tm(s, 3); if (lin_chunked && kr_sv_lin_scan_wide_fits(q.kind, q.dim)) kr_sv_lin_scan_wide(q, st); else kr_sv_lin_scan(q, st); }
             KrSvSsdOut so{};
             so.o = (const float*)s->lin_o.p; so.x = (const float*)s->sconv.p; so.ld_x = cc; so.z = zin; so.ld_z = l.n_h; so.D = (const float*)l.ssd_d.p; so.w = (const float*)l.ssd_norm.p;
             so.heads = d.ssd_heads; so.vdim = d.ssd_vdim; so.groups = d.ssd_norm_groups; so.eps = c.norm_eps;

@@ -1181,6 +1181,135 @@ __global__ void __launch_bounds__(64) sv_lin_scan_kernel(const KrSvLin a) {
     if (ML && lane == 0) nmg[dim] = m;
 }
 
+// Prompt portions of the gla and state-space mixers (kinds 4, 5): the same recurrence, token by token, laid out for the length of the serial chain.
+// One WORKGROUP of four waves per (request, head, block of 16 value columns); a wave owns 4 columns, lane = 16 * column + part, and a lane keeps the rows
+// [part * dpr, (part + 1) * dpr) of its column of S in registers (dpr = ceil(dim / 16) <= DP): a token costs a lane dpr updates and dpr products, and the
+// sixteen parts of a column meet in four lane exchanges inside their row of 16 lanes.  The chain of a head is thus spread over 8 times as many lanes
+// as in sv_lin_scan_kernel, and the compute units the short grid leaves idle take them.  Tokens are staged 16 at a time in one of two LDS buffers:
+// the loads of the next 16 are issued before the current 16 are walked and land in registers meanwhile (one barrier per 16 tokens).  With 16 tokens
+// of 16 * dpr rows a thread stages exactly dpr elements of q, of k and of the decays per batch.  a.gz holds the decays themselves (sv_gla_decay_kernel).
+template <int KIND, int DP>
+__global__ void __launch_bounds__(256) sv_lin_scanw_kernel(const KrSvLin a) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int TB = 16;
+    constexpr bool GLA = KIND == 4, SSD = KIND == 5;
+    const int e = blockIdx.x, h = blockIdx.y, cb = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int part = lane & 15, cl = wave * 4 + (lane >> 4), col = cb * 16 + cl;
+    const int dim = a.dim, vdim = a.vdim, H = a.heads;
+    const int dpr = (dim + 15) / 16, dimp = 16 * dpr;
+    const int t0 = a.ent_off[e], t1 = a.ent_off[e + 1], sl = a.ent_slot[e];
+    const bool fresh = a.pos[t0] == 0, cv = col < vdim;
+    float* Sg = a.state + (size_t)sl * a.state_stride + ((size_t)h * vdim + (cv ? col : 0)) * dim + part * dpr;
+    float S[DP];
+#pragma unroll
+    for (int r = 0; r < DP; r++) S[r] = (r < dpr && part * dpr + r < dim && !fresh && cv) ? Sg[r] : 0.0f;
+    const int per = (GLA ? 3 : 2) * TB * dimp + TB * 16 + TB * 2;      // floats of one buffer: q | k | (decays) | v | gates
+    const int hq = h / a.qk_group;
+    // staging: thread (token tid / 16 of the batch, column tid % 16 + 16 j of the row) -- dpr elements of q, of k and of the decays per thread and batch.
+    // fetch() is loads and nothing else (clamped addresses, no use of a loaded value), so that no wait stands between it and the walk over the current
+    // batch; scales, masks and the gates' functions are applied when the registers go to LDS
+    float pq[DP], pk[DP], pa[DP], pv = 0.0f, pg = 0.0f;
+    const int ft = tid >> 4, fd = tid & 15;
+    auto fetch = [&](int tb) {               // global -> registers
+        const int nt = min(TB, t1 - tb), tok = tb + min(ft, nt - 1);
+        const size_t rb = (size_t)tok * a.src_ld + (size_t)hq * dim;
+#pragma unroll
+        for (int j = 0; j < DP; j++) {
+            if (j < dpr) {
+                const int d = min(fd + 16 * j, dim - 1);
+                pq[j] = a.qsrc[rb + d]; pk[j] = a.ksrc[rb + d];
+                if constexpr (GLA) pa[j] = a.gz[(size_t)tok * a.gz_ld + (size_t)h * dim + d];
+            }
+        }
+        pv = a.vsrc[(size_t)tok * a.src_ld + (size_t)h * vdim + min(cb * 16 + fd, vdim - 1)];
+        if constexpr (SSD) pg = a.dtz[(size_t)(tb + min(tid, nt - 1)) * a.dtz_ld + h];
+    };
+    const float ssd_rate = SSD ? -expf(a.a_log[h]) : 0.0f, ssd_bias = SSD ? a.dt_bias[h] : 0.0f;
+    auto stash = [&](float* buf, int tb) {   // registers -> LDS
+        const int nt = min(TB, t1 - tb);
+        float* qs = buf; float* ks = qs + TB * dimp; float* as = ks + TB * dimp; float* vs = buf + (GLA ? 3 : 2) * TB * dimp; float* gs = vs + TB * 16;
+#pragma unroll
+        for (int j = 0; j < DP; j++)
+            if (j < dpr) {
+                const int d = fd + 16 * j, idx = ft * dimp + d;
+                const bool ok = ft < nt && d < dim;
+                qs[idx] = ok ? pq[j] * a.q_scale : 0.0f; ks[idx] = ok ? pk[j] * a.k_scale : 0.0f;
+                if constexpr (GLA) as[idx] = ok ? pa[j] : 0.0f;
+            }
+        vs[tid] = (ft < nt && cb * 16 + fd < vdim) ? pv : 0.0f;
+        if (SSD && tid < TB) {
+            const float z = pg + ssd_bias;
+            const float dt = fmaxf(z, 0.0f) + log1pf(expf(-fabsf(z)));      // softplus
+            gs[2 * tid] = dt; gs[2 * tid + 1] = expf(ssd_rate * dt);
+        }
+    };
+    fetch(t0); stash(lds, t0);
+    __syncthreads();
+    int b = 0;
+    for (int tb = t0; tb < t1; tb += TB, b ^= 1) {
+        const int nt = min(TB, t1 - tb);
+        const bool more = tb + TB < t1;
+        if (more) fetch(tb + TB);
+        const float* buf = lds + b * per;
+        const float* qs = buf; const float* ks = qs + TB * dimp; const float* as = ks + TB * dimp; const float* vs = buf + (GLA ? 3 : 2) * TB * dimp; const float* gs = vs + TB * 16;
+        // one token: the lane's rows of q, k and the decays come from LDS (16-byte reads when the lane's rows fill DP), the state stays in registers
+        auto token = [&](int tt) -> float {
+            const float* qp = qs + tt * dimp + part * dpr; const float* kp = ks + tt * dimp + part * dpr; const float* ap = as + tt * dimp + part * dpr;
+            float qv[DP], kv[DP], dv[DP];
+            if (dpr == DP) {
+#pragma unroll
+                for (int r = 0; r < DP; r += 4) {
+                    const float4 q4 = *reinterpret_cast<const float4*>(qp + r), k4 = *reinterpret_cast<const float4*>(kp + r);
+                    qv[r] = q4.x; qv[r + 1] = q4.y; qv[r + 2] = q4.z; qv[r + 3] = q4.w; kv[r] = k4.x; kv[r + 1] = k4.y; kv[r + 2] = k4.z; kv[r + 3] = k4.w;
+                    if constexpr (GLA) { const float4 a4 = *reinterpret_cast<const float4*>(ap + r); dv[r] = a4.x; dv[r + 1] = a4.y; dv[r + 2] = a4.z; dv[r + 3] = a4.w; }
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < DP; r++) { qv[r] = r < dpr ? qp[r] : 0.0f; kv[r] = r < dpr ? kp[r] : 0.0f; if constexpr (GLA) dv[r] = r < dpr ? ap[r] : 0.0f; }
+            }
+            float av = 1.0f, bvv = vs[tt * 16 + cl];
+            if constexpr (SSD) { bvv *= gs[2 * tt]; av = gs[2 * tt + 1]; }
+            float po0 = 0.0f, po1 = 0.0f;
+#pragma unroll
+            for (int r = 0; r < DP; r += 2) {
+                if constexpr (GLA) { S[r] = __builtin_fmaf(kv[r], bvv, dv[r] * S[r]); S[r + 1] = __builtin_fmaf(kv[r + 1], bvv, dv[r + 1] * S[r + 1]); }
+                else { S[r] = __builtin_fmaf(kv[r], bvv, av * S[r]); S[r + 1] = __builtin_fmaf(kv[r + 1], bvv, av * S[r + 1]); }
+                po0 = __builtin_fmaf(S[r], qv[r], po0); po1 = __builtin_fmaf(S[r + 1], qv[r + 1], po1);
+            }
+            float po = po0 + po1;
+            po += SV_DPPF(po, KR_DPP_XOR1); po += SV_DPPF(po, KR_DPP_XOR2); po += SV_DPPF(po, KR_DPP_HALF_MIRROR); po += SV_DPPF(po, KR_DPP_MIRROR);
+            return po;
+        };
+        // the batch's outputs stay in registers and leave after the loop: the loop body has no branch, so the LDS reads of the next tokens are issued while
+        // the current one is worked on
+        float outv[TB];
+        if (nt == TB) {
+#pragma unroll
+            for (int tt = 0; tt < TB; tt++) outv[tt] = token(tt);
+        } else {
+#pragma unroll
+            for (int tt = 0; tt < TB; tt++) outv[tt] = tt < nt ? token(tt) : 0.0f;
+        }
+        if (part == 0 && cv) {
+            float* op = a.o + (size_t)tb * H * vdim + (size_t)h * vdim + col;
+#pragma unroll
+            for (int tt = 0; tt < TB; tt++) if (tt < nt) op[(size_t)tt * H * vdim] = outv[tt];
+        }
+        if (more) stash(lds + (b ^ 1) * per, tb + TB);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int r = 0; r < DP; r++)
+        if (r < dpr && part * dpr + r < dim && cv) Sg[r] = S[r];
+}
+// gla: the decays themselves from their logits, in place: a = sigmoid(z + b)^(1 / tau), formed through the logarithm
+__global__ void sv_gla_decay_kernel(float* __restrict__ gz, const float* __restrict__ bias, size_t n, int cols, float inv_tau) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float z = gz[i] + bias[i % cols];
+    gz[i] = expf((fminf(z, 0.0f) - log1pf(expf(-fabsf(z)))) * inv_tau);
+}
+
 // ---- chunked form for prompt portions (KrSvLin: tok, sbuf, nbuf)
 // rotation and scales on q / k in place, and the log gates of every (token, head): tok.x = log decay a, tok.y = log input b
 __global__ void __launch_bounds__(64) sv_lin_prep_kernel(const KrSvLin a) {
@@ -1769,6 +1898,25 @@ void kr_sv_lin_scan(const KrSvLin& a, hipStream_t st) {
     if (a.kind == 3) SV_LIN_D(3); else if (a.kind == 4) SV_LIN_D(4); else if (a.kind == 5) SV_LIN_D(5); else SV_LIN_D(2);
 #undef SV_LIN_D
 #undef SV_LIN
+}
+// the workgroup form for prompt portions of kinds 4 and 5; false: the shape does not fit its LDS buffers (the caller takes kr_sv_lin_scan)
+static size_t sv_scanw_lds(int kind, int dim) { const int dimp = 16 * ((dim + 15) / 16); return (size_t)2 * ((kind == 4 ? 3 : 2) * 16 * dimp + 16 * 16 + 16 * 2) * sizeof(float); }
+bool kr_sv_lin_scan_wide_fits(int kind, int dim) { return (kind == 4 || kind == 5) && dim <= 512 && sv_scanw_lds(kind, dim) <= 150 * 1024; }
+void kr_sv_lin_scan_wide(const KrSvLin& a, hipStream_t st) {
+    if (a.T <= 0 || a.n_entries <= 0) return;
+    const int dpr = (a.dim + 15) / 16;
+    const dim3 grid(a.n_entries, a.heads, (a.vdim + 15) / 16);
+    const size_t lds = sv_scanw_lds(a.kind, a.dim);
+    if (a.kind == 4) {
+        const size_t n = (size_t)a.T * a.heads * a.dim;
+        hipLaunchKernelGGL(sv_gla_decay_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, const_cast<float*>(a.gz), a.gz_bias, n, a.heads * a.dim, a.inv_tau);
+    }
+#define SV_LW(K_, DP_) do { if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)sv_lin_scanw_kernel<K_, DP_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+                            hipLaunchKernelGGL((sv_lin_scanw_kernel<K_, DP_>), grid, dim3(256), lds, st, a); } while (0)
+#define SV_LW_D(K_) do { if (dpr <= 4) SV_LW(K_, 4); else if (dpr <= 8) SV_LW(K_, 8); else if (dpr <= 16) SV_LW(K_, 16); else SV_LW(K_, 32); } while (0)
+    if (a.kind == 4) SV_LW_D(4); else SV_LW_D(5);
+#undef SV_LW_D
+#undef SV_LW
 }
 bool kr_sv_lin_chunked_fits(int dim, int vdim) { return dim <= 128 && vdim <= 128; }
 void kr_sv_lin_chunked(const KrSvLin& a, hipStream_t st) {

@@ -2,7 +2,8 @@
     python tools/probes/serve_profile.py <small|large> prefill [design]     three prompt passes of the size's prompt length
     python tools/probes/serve_profile.py <small|large> decode [design]      decode steps of 1 and of 4 requests at the end of such a prompt, graphs on / off
 design: lomutar (default), pamulix:<one letter per layer, A = chunked attention, L = attention through latents>, e.g. pamulix:ALAA, or
-midisun:<A = windowed attention, R = retention, M = mLSTM>, e.g. midisun:ARMA
+midisun:<A = windowed attention, R = retention, M = mLSTM>, e.g. midisun:ARMA, or lufozen:<A = attention, P = attention beside a state-space mixer, G = gla>, e.g.
+lufozen:APGA (the second and third layer run twice)
 Run under `rocprofv3 --kernel-trace --stats` for the kernel tables in profiles/serve_*."""
 import os
 import sys
@@ -25,6 +26,8 @@ if design.startswith("pamulix:"):
     eng = bench.pamulix_serve_engine(z, design.split(":", 1)[1])
 elif design.startswith("midisun:"):
     eng = bench.midisun_serve_engine(z, design.split(":", 1)[1])
+elif design.startswith("lufozen:"):
+    eng, _ = bench.lufozen_serve_engine(z, design.split(":", 1)[1], k * F)
 else:
     eng = SCH.BatchEngine(R.ServeModelSpec(V, W, S.NORM_LAYER, 1e-5, layers, None), dtype="bfloat16", max_tokens=4 * (P + 256), max_slots=4)
     eng.load_synthetic(seed=7, amp=1.0)
