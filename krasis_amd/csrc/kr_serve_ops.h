@@ -203,7 +203,7 @@ void kr_sv_lin_scan(const KrSvLin& a, hipStream_t st);
 // prompt portions in blocks of 64 tokens on the f32 matrix instruction (rotation and scales applied to q / k in place first): within a block
 // o_t = g_t S_start^T q_t + sum_(s <= t) exp(u_t + w_s) (q_t . k_s) v_s, and S_end = g_last S_start + sum_s exp(u_last + w_s) k_s v_s^T; a short serial
 // launch carries S from block to block, the outputs of all blocks are formed in parallel.  Same state layout as kr_sv_lin_scan.
-// kinds 4 and 5, prompt portions: a workgroup per (request, head, 16 value columns), the rows of S spread over sixteen lanes per column, tokens staged
+// kinds 4 and 5, prompt portions: a workgroup per (request, head, 8 value columns), the rows of S spread over thirty-two lanes per column, tokens staged
 // sixteen at a time through two LDS buffers.  For kind 4 the launcher first turns a.gz (written by the caller, logits) into the decays, in place.
 bool kr_sv_lin_scan_wide_fits(int kind, int dim);
 void kr_sv_lin_scan_wide(const KrSvLin& a, hipStream_t st);

@@ -1181,62 +1181,65 @@ __global__ void __launch_bounds__(64) sv_lin_scan_kernel(const KrSvLin a) {
     if (ML && lane == 0) nmg[dim] = m;
 }
 
-// Prompt portions of the gla and state-space mixers (kinds 4, 5): the same recurrence, token by token, laid out for the length of the serial chain.
-// One WORKGROUP of four waves per (request, head, block of 16 value columns); a wave owns 4 columns, lane = 16 * column + part, and a lane keeps the rows
-// [part * dpr, (part + 1) * dpr) of its column of S in registers (dpr = ceil(dim / 16) <= DP): a token costs a lane dpr updates and dpr products, and the
-// sixteen parts of a column meet in four lane exchanges inside their row of 16 lanes.  The chain of a head is thus spread over 8 times as many lanes
-// as in sv_lin_scan_kernel, and the compute units the short grid leaves idle take them.  Tokens are staged 16 at a time in one of two LDS buffers:
-// the loads of the next 16 are issued before the current 16 are walked and land in registers meanwhile (one barrier per 16 tokens).  With 16 tokens
-// of 16 * dpr rows a thread stages exactly dpr elements of q, of k and of the decays per batch.  a.gz holds the decays themselves (sv_gla_decay_kernel).
+// Prompt portions of the gla and state-space mixers (kinds 4, 5): the same recurrence, token by token, laid out for the length of the serial chain:
+// what a portion waits for is the instructions ONE wave issues per token, so a head's state is spread over as many lanes as the chip has to spare.
+// One WORKGROUP of four waves per (request, head, block of 8 value columns); a wave owns 2 columns, lane = 32 * column + part, and a lane keeps the rows
+// [part * dpr, (part + 1) * dpr) of its column of S in registers (dpr = ceil(dim / 32) <= DP): a token costs a lane dpr updates and dpr products, and the
+// thirty-two parts of a column meet in four exchanges inside their rows of 16 lanes and one across the two rows.  Tokens are staged 16 at a time in one
+// of two LDS buffers: the loads of the next 16 are issued before the current 16 are walked and land in registers meanwhile (one barrier per 16
+// tokens); the walk itself has no branch and no store (the 16 outputs of a lane leave together afterwards), so the LDS reads of the following tokens
+// are in flight while one is worked on.  a.gz holds the decays themselves (sv_gla_decay_kernel).
 template <int KIND, int DP>
 __global__ void __launch_bounds__(256) sv_lin_scanw_kernel(const KrSvLin a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
-    constexpr int TB = 16;
+    constexpr int TB = 16, NC = 8;           // tokens per batch, value columns per workgroup
     constexpr bool GLA = KIND == 4, SSD = KIND == 5;
     const int e = blockIdx.x, h = blockIdx.y, cb = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int part = lane & 15, cl = wave * 4 + (lane >> 4), col = cb * 16 + cl;
+    const int part = lane & 31, cl = wave * 2 + (lane >> 5), col = cb * NC + cl;
     const int dim = a.dim, vdim = a.vdim, H = a.heads;
-    const int dpr = (dim + 15) / 16, dimp = 16 * dpr;
+    // a lane's dpr rows stand together in LDS, the parts of a token `pitch` floats apart: dpr + 4 where dpr is a multiple of 8, so that the 16-byte reads of
+    // neighbouring parts fall into distinct banks
+    const int dpr = (dim + 31) / 32, pitch = (dpr % 8 == 0) ? dpr + 4 : dpr, dimp = 32 * pitch;
     const int t0 = a.ent_off[e], t1 = a.ent_off[e + 1], sl = a.ent_slot[e];
     const bool fresh = a.pos[t0] == 0, cv = col < vdim;
     float* Sg = a.state + (size_t)sl * a.state_stride + ((size_t)h * vdim + (cv ? col : 0)) * dim + part * dpr;
     float S[DP];
 #pragma unroll
     for (int r = 0; r < DP; r++) S[r] = (r < dpr && part * dpr + r < dim && !fresh && cv) ? Sg[r] : 0.0f;
-    const int per = (GLA ? 3 : 2) * TB * dimp + TB * 16 + TB * 2;      // floats of one buffer: q | k | (decays) | v | gates
+    const int per = (GLA ? 3 : 2) * TB * dimp + TB * NC + TB * 2;      // floats of one buffer: q | k | (decays) | v | gates
     const int hq = h / a.qk_group;
-    // staging: thread (token tid / 16 of the batch, column tid % 16 + 16 j of the row) -- dpr elements of q, of k and of the decays per thread and batch.
+    // staging: thread (token tid / 16 of the batch, row tid % 16 + 16 j of the head) -- 2 dpr elements of q, of k and of the decays per thread and batch.
     // fetch() is loads and nothing else (clamped addresses, no use of a loaded value), so that no wait stands between it and the walk over the current
     // batch; scales, masks and the gates' functions are applied when the registers go to LDS
-    float pq[DP], pk[DP], pa[DP], pv = 0.0f, pg = 0.0f;
+    float pq[2 * DP], pk[2 * DP], pa[2 * DP], pv = 0.0f, pg = 0.0f;
     const int ft = tid >> 4, fd = tid & 15;
     auto fetch = [&](int tb) {               // global -> registers
         const int nt = min(TB, t1 - tb), tok = tb + min(ft, nt - 1);
         const size_t rb = (size_t)tok * a.src_ld + (size_t)hq * dim;
 #pragma unroll
-        for (int j = 0; j < DP; j++) {
-            if (j < dpr) {
+        for (int j = 0; j < 2 * DP; j++) {
+            if (j < 2 * dpr) {
                 const int d = min(fd + 16 * j, dim - 1);
                 pq[j] = a.qsrc[rb + d]; pk[j] = a.ksrc[rb + d];
                 if constexpr (GLA) pa[j] = a.gz[(size_t)tok * a.gz_ld + (size_t)h * dim + d];
             }
         }
-        pv = a.vsrc[(size_t)tok * a.src_ld + (size_t)h * vdim + min(cb * 16 + fd, vdim - 1)];
+        pv = a.vsrc[(size_t)(tb + min(tid >> 3, nt - 1)) * a.src_ld + (size_t)h * vdim + min(cb * NC + (tid & 7), vdim - 1)];      // threads below 128: (token, column)
         if constexpr (SSD) pg = a.dtz[(size_t)(tb + min(tid, nt - 1)) * a.dtz_ld + h];
     };
     const float ssd_rate = SSD ? -expf(a.a_log[h]) : 0.0f, ssd_bias = SSD ? a.dt_bias[h] : 0.0f;
     auto stash = [&](float* buf, int tb) {   // registers -> LDS
         const int nt = min(TB, t1 - tb);
-        float* qs = buf; float* ks = qs + TB * dimp; float* as = ks + TB * dimp; float* vs = buf + (GLA ? 3 : 2) * TB * dimp; float* gs = vs + TB * 16;
+        float* qs = buf; float* ks = qs + TB * dimp; float* as = ks + TB * dimp; float* vs = buf + (GLA ? 3 : 2) * TB * dimp; float* gs = vs + TB * NC;
 #pragma unroll
-        for (int j = 0; j < DP; j++)
-            if (j < dpr) {
-                const int d = fd + 16 * j, idx = ft * dimp + d;
+        for (int j = 0; j < 2 * DP; j++)
+            if (j < 2 * dpr) {
+                const int d = fd + 16 * j, pp = dpr == DP ? d / DP : d / dpr, idx = ft * dimp + pp * pitch + (d - pp * dpr);
                 const bool ok = ft < nt && d < dim;
                 qs[idx] = ok ? pq[j] * a.q_scale : 0.0f; ks[idx] = ok ? pk[j] * a.k_scale : 0.0f;
                 if constexpr (GLA) as[idx] = ok ? pa[j] : 0.0f;
             }
-        vs[tid] = (ft < nt && cb * 16 + fd < vdim) ? pv : 0.0f;
+        if (tid < TB * NC) vs[tid] = ((tid >> 3) < nt && cb * NC + (tid & 7) < vdim) ? pv : 0.0f;
         if (SSD && tid < TB) {
             const float z = pg + ssd_bias;
             const float dt = fmaxf(z, 0.0f) + log1pf(expf(-fabsf(z)));      // softplus
@@ -1251,10 +1254,10 @@ __global__ void __launch_bounds__(256) sv_lin_scanw_kernel(const KrSvLin a) {
         const bool more = tb + TB < t1;
         if (more) fetch(tb + TB);
         const float* buf = lds + b * per;
-        const float* qs = buf; const float* ks = qs + TB * dimp; const float* as = ks + TB * dimp; const float* vs = buf + (GLA ? 3 : 2) * TB * dimp; const float* gs = vs + TB * 16;
+        const float* qs = buf; const float* ks = qs + TB * dimp; const float* as = ks + TB * dimp; const float* vs = buf + (GLA ? 3 : 2) * TB * dimp; const float* gs = vs + TB * NC;
         // one token: the lane's rows of q, k and the decays come from LDS (16-byte reads when the lane's rows fill DP), the state stays in registers
         auto token = [&](int tt) -> float {
-            const float* qp = qs + tt * dimp + part * dpr; const float* kp = ks + tt * dimp + part * dpr; const float* ap = as + tt * dimp + part * dpr;
+            const float* qp = qs + tt * dimp + part * pitch; const float* kp = ks + tt * dimp + part * pitch; const float* ap = as + tt * dimp + part * pitch;
             float qv[DP], kv[DP], dv[DP];
             if (dpr == DP) {
 #pragma unroll
@@ -1267,7 +1270,7 @@ __global__ void __launch_bounds__(256) sv_lin_scanw_kernel(const KrSvLin a) {
 #pragma unroll
                 for (int r = 0; r < DP; r++) { qv[r] = r < dpr ? qp[r] : 0.0f; kv[r] = r < dpr ? kp[r] : 0.0f; if constexpr (GLA) dv[r] = r < dpr ? ap[r] : 0.0f; }
             }
-            float av = 1.0f, bvv = vs[tt * 16 + cl];
+            float av = 1.0f, bvv = vs[tt * NC + cl];
             if constexpr (SSD) { bvv *= gs[2 * tt]; av = gs[2 * tt + 1]; }
             float po0 = 0.0f, po1 = 0.0f;
 #pragma unroll
@@ -1278,10 +1281,8 @@ __global__ void __launch_bounds__(256) sv_lin_scanw_kernel(const KrSvLin a) {
             }
             float po = po0 + po1;
             po += SV_DPPF(po, KR_DPP_XOR1); po += SV_DPPF(po, KR_DPP_XOR2); po += SV_DPPF(po, KR_DPP_HALF_MIRROR); po += SV_DPPF(po, KR_DPP_MIRROR);
-            return po;
+            return po + __shfl_xor(po, 16);
         };
-        // the batch's outputs stay in registers and leave after the loop: the loop body has no branch, so the LDS reads of the next tokens are issued while
-        // the current one is worked on
         float outv[TB];
         if (nt == TB) {
 #pragma unroll
@@ -1290,12 +1291,13 @@ __global__ void __launch_bounds__(256) sv_lin_scanw_kernel(const KrSvLin a) {
 #pragma unroll
             for (int tt = 0; tt < TB; tt++) outv[tt] = tt < nt ? token(tt) : 0.0f;
         }
+        if (more) stash(lds + (b ^ 1) * per, tb + TB);
+        // the outputs leave after the registers of the next batch have gone to LDS: the wait for those loads then has no younger store before it
         if (part == 0 && cv) {
             float* op = a.o + (size_t)tb * H * vdim + (size_t)h * vdim + col;
 #pragma unroll
             for (int tt = 0; tt < TB; tt++) if (tt < nt) op[(size_t)tt * H * vdim] = outv[tt];
         }
-        if (more) stash(lds + (b ^ 1) * per, tb + TB);
         __syncthreads();
     }
 #pragma unroll
@@ -1900,12 +1902,15 @@ void kr_sv_lin_scan(const KrSvLin& a, hipStream_t st) {
 #undef SV_LIN
 }
 // the workgroup form for prompt portions of kinds 4 and 5; false: the shape does not fit its LDS buffers (the caller takes kr_sv_lin_scan)
-static size_t sv_scanw_lds(int kind, int dim) { const int dimp = 16 * ((dim + 15) / 16); return (size_t)2 * ((kind == 4 ? 3 : 2) * 16 * dimp + 16 * 16 + 16 * 2) * sizeof(float); }
+static size_t sv_scanw_lds(int kind, int dim) {
+    const int dpr = (dim + 31) / 32, dimp = 32 * ((dpr % 8 == 0) ? dpr + 4 : dpr);
+    return (size_t)2 * ((kind == 4 ? 3 : 2) * 16 * dimp + 16 * 8 + 16 * 2) * sizeof(float);
+}
 bool kr_sv_lin_scan_wide_fits(int kind, int dim) { return (kind == 4 || kind == 5) && dim <= 512 && sv_scanw_lds(kind, dim) <= 150 * 1024; }
 void kr_sv_lin_scan_wide(const KrSvLin& a, hipStream_t st) {
     if (a.T <= 0 || a.n_entries <= 0) return;
-    const int dpr = (a.dim + 15) / 16;
-    const dim3 grid(a.n_entries, a.heads, (a.vdim + 15) / 16);
+    const int dpr = (a.dim + 31) / 32;
+    const dim3 grid(a.n_entries, a.heads, (a.vdim + 7) / 8);
     const size_t lds = sv_scanw_lds(a.kind, a.dim);
     if (a.kind == 4) {
         const size_t n = (size_t)a.T * a.heads * a.dim;
@@ -1913,7 +1918,7 @@ void kr_sv_lin_scan_wide(const KrSvLin& a, hipStream_t st) {
     }
 #define SV_LW(K_, DP_) do { if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)sv_lin_scanw_kernel<K_, DP_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
                             hipLaunchKernelGGL((sv_lin_scanw_kernel<K_, DP_>), grid, dim3(256), lds, st, a); } while (0)
-#define SV_LW_D(K_) do { if (dpr <= 4) SV_LW(K_, 4); else if (dpr <= 8) SV_LW(K_, 8); else if (dpr <= 16) SV_LW(K_, 16); else SV_LW(K_, 32); } while (0)
+#define SV_LW_D(K_) do { if (dpr <= 4) SV_LW(K_, 4); else if (dpr <= 8) SV_LW(K_, 8); else SV_LW(K_, 16); } while (0)
     if (a.kind == 4) SV_LW_D(4); else SV_LW_D(5);
 #undef SV_LW_D
 #undef SV_LW
