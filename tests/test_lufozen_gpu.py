@@ -533,3 +533,35 @@ def test_graph_replays_equal_eager_steps():
     ref = O.forward(cfg, {k: O.bf16_round(v) for k, v in W.items()}, a[:131])[0]
     e = np.sqrt(((lg[0] - ref[130]) ** 2).mean()) / np.sqrt((ref ** 2).mean())
     assert e < 5e-2
+
+
+def test_state_space_mixer_as_a_layers_only_mixer():
+    """the store's state-space mixer without an attention beside it (no registered design asks for that; another one may): plain RMS norms, no pair table"""
+    from krasis_amd import model_registry as R, serve_store as S
+    from krasis_amd.scheduler import BatchEngine
+    rng = np.random.default_rng(3)
+    width, vocab, m = 48, 30, O.ssd(3, 10, 6, groups=3, conv=3, norm_groups=2)
+    cfgw = O.random_weights(small_model([O.layer(O.parallel(O.left(1, 1, 4, 4), m), None)], width=width, vocab=vocab), 9)
+    W = {k: v for k, v in cfgw.items() if k.startswith("l0.mix.right.") or k in ("embed", "head")}
+    W["l0.norm1"] = (1.0 + 0.1 * rng.standard_normal(width)).astype(np.float32); W["final.norm"] = (1.0 + 0.1 * rng.standard_normal(width)).astype(np.float32)
+
+    def names(spec):
+        yield -1, "embed", 0, "embed"
+        yield -1, "final_norm_w", 0, "final.norm"
+        yield -1, "head", 0, "head"
+        yield 0, "norm_w", 0, "l0.norm1"
+        for role, n in (("ssd_in", "in"), ("ssd_conv", "conv"), ("ssd_conv_b", "conv.b"), ("ssd_dt_bias", "dt_bias"), ("ssd_a_log", "A_log"), ("ssd_d", "D"), ("ssd_norm", "norm"), ("ssd_o", "o")):
+            yield 0, role, 0, "l0.mix.right." + n
+    layer = S.LayerSpec(heads=1, kv_heads=1, dim=1, vdim=1, mixer_kind=S.MIX_SSD, ssd_heads=3, ssd_vdim=10, ssd_state=6, ssd_groups=3, ssd_conv=3, ssd_norm_groups=2)
+    spec = R.ServeModelSpec(vocab, width, S.NORM_RMS, 1e-5, [layer], names, block_kind=S.BLOCK_SEQUENTIAL, pre_norm=1, post_norm=0, norm_bias=0)
+    eng = BatchEngine(spec, dtype="float32", max_tokens=256)
+    eng.load_arrays(W)
+    toks = [int(t) for t in rng.integers(0, vocab, 50)]
+    w64 = {k: v.astype(np.float64) for k, v in W.items()}
+    x = w64["embed"][toks]
+    x = x + O.mixer_ssd(m, w64, "l0.mix.right.", O.rms_unit(x, 1e-5) * w64["l0.norm1"], 1e-5)
+    ref = (O.rms_unit(x, 1e-5) * w64["final.norm"]) @ w64["head"].T
+    whole, _ = eng.step([("w", toks, list(range(50)))])
+    assert rel(whole, ref) < 2e-4
+    rows = [eng.step([("d", toks[:7], [6])])[0][0]] + [eng.step([("d", [t], [0])])[0][0] for t in toks[7:]]
+    assert rel(np.stack(rows), ref[6:]) < 2e-4
