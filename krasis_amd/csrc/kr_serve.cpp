@@ -84,6 +84,7 @@ struct kr_serve {
     // f32 copy of the mixer's normed input, its convolved form, residual gate logits, whole-row q / k statistics, recurrent outputs; chunked recurrence:
     // per-token gate terms, state / normaliser at every block's start, per-block gate terms
     DevBuf h32, hc, rg, qk_rms, lin_o, lin_tok, lin_sbuf, lin_nbuf, lin_cm;
+    DevBuf ssd_z;                                         // the state-space mixer's rows in the block recurrence's layout [q | k | v] per head (prompt portions)
     DevBuf qkv2, sconv, ga1, gz;                          // convolved q | k | v; convolved x | B | C; the gla decay's low-rank input (storage type) and logits
     DevBuf v_first;                                      // [T, kv_heads * vdim] f32: the values of the first value-mixing layer
     DevBuf lq_c, lq_2, lq_n, lq_e, att2, head_i;         // latent mixer: query latent, W_uq output, plain query parts, folded queries, per-head values, head row tables
@@ -831,13 +832,19 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
     const bool seq = c.block_kind == KR_SERVE_BLOCK_SEQUENTIAL;
     size_t max_qkv = 0, max_att = 0, max_gu = 0, max_y = 0, max_rows = 0, max_pairs = 0, max_vf = 0; int max_E = 1;
     size_t lq_c = 0, lq_2 = 0, lq_n = 0, lq_e = 0, att2 = 0, head_i = 0, max_lin = 0, lin_tok = 0, lin_sb = 0, lin_nb = 0; bool whole_norm = false;
-    size_t max_pconv = 0, max_sconv = 0, max_ga1 = 0, max_gz = 0;
+    size_t max_pconv = 0, max_sconv = 0, max_ga1 = 0, max_gz = 0, max_ssdz = 0;
     // prompt portions take the chunked form of the recurrent mixers (blocks of 64 tokens on the matrix instruction), decode-sized steps the token-by-token form
     const bool lin_chunked = max_count >= 32;
     for (const SvLayer& l : s->L) {
         const kr_serve_layer& d = l.d;
         if (d.proj_conv) max_pconv = std::max(max_pconv, (size_t)l.pconv_c());
-        if (l.has_ssd()) { max_sconv = std::max(max_sconv, (size_t)l.ssd_conv_c()); max_lin = std::max(max_lin, (size_t)l.ssd_inner()); }
+        if (l.has_ssd()) {
+            max_sconv = std::max(max_sconv, (size_t)l.ssd_conv_c()); max_lin = std::max(max_lin, (size_t)l.ssd_inner());
+            if (lin_chunked && kr_sv_lin_chunked_fits(d.ssd_state, d.ssd_vdim)) {
+                lin_tok = std::max(lin_tok, (size_t)d.ssd_heads); lin_sb = std::max(lin_sb, (size_t)d.ssd_heads * d.ssd_state * d.ssd_vdim); lin_nb = std::max(lin_nb, (size_t)d.ssd_heads * d.ssd_state);
+                max_ssdz = std::max(max_ssdz, (size_t)d.ssd_heads * (2 * d.ssd_state + d.ssd_vdim));
+            }
+        }
         if (l.gla()) { max_ga1 = std::max(max_ga1, (size_t)d.decay_rank); max_gz = std::max(max_gz, (size_t)d.heads * d.dim); }
         if (l.recurrent()) {
             max_lin = std::max(max_lin, (size_t)d.heads * d.vdim);
@@ -875,6 +882,7 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         return kr_fail(KR_ERR_HIP, "block scratch for %d tokens", T);
     if ((max_pconv && s->qkv2.ensure(Ts * max_pconv * 4)) || (max_sconv && s->sconv.ensure(Ts * max_sconv * 4)) || (max_ga1 && (s->ga1.ensure(Ts * max_ga1 * s->esz) || s->gz.ensure(Ts * max_gz * 4))))
         return kr_fail(KR_ERR_HIP, "convolution / decay scratch for %d tokens", T);
+    if (max_ssdz && s->ssd_z.ensure(Ts * max_ssdz * 4)) return kr_fail(KR_ERR_HIP, "state-space block scratch for %d tokens", T);
     for (SvRope& r : s->ropes) if (r.cs.ensure(Ts * (r.dims / 2) * 8)) return kr_fail(KR_ERR_HIP, "rope table");
     if (s->capture) { if (s->cap.ensure((size_t)c.n_layers * Ts * W * 4)) return kr_fail(KR_ERR_HIP, "capture buffer"); s->cap_T = T; }
     std::vector<int> nsplit(c.n_layers, 1);
@@ -1071,7 +1079,22 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
             q.dtz = zin + inner + cc; q.dtz_ld = l.n_h; q.dt_bias = (const float*)l.dt_bias.p; q.a_log = (const float*)l.a_log.p;
             q.state = (float*)run.ssd_state.p; q.state_stride = l.ssd_state_stride;
             q.ent_off = d_eoff; q.ent_slot = d_eslot; q.n_entries = n_entries; q.pos = d_pos; q.T = T; q.o = (float*)s->lin_o.p;
-            { Timer tm(s, 3); if (lin_chunked && kr_sv_lin_scan_wide_fits(q.kind, q.dim)) kr_sv_lin_scan_wide(q, st); else kr_sv_lin_scan(q, st); }
+            {
+                Timer tm(s, 3);
+                if (lin_chunked && kr_sv_lin_chunked_fits(d.ssd_state, d.ssd_vdim)) {
+                    // prompt portions: a retention with a decay per token, on the block launches of the recurrent mixers (same state layout)
+                    const int ldz = d.ssd_heads * (2 * d.ssd_state + d.ssd_vdim);
+                    q.tok = (float4*)s->lin_tok.p;
+                    kr_sv_ssd_expand(q, (float*)s->ssd_z.p, ldz, st);
+                    KrSvLin c2{};
+                    c2.kind = KR_SERVE_MIX_RETENTION; c2.prepped = 1; c2.z = (float*)s->ssd_z.p; c2.ld = ldz; c2.heads = d.ssd_heads; c2.dim = d.ssd_state; c2.vdim = d.ssd_vdim;
+                    c2.q_scale = c2.k_scale = 1.0f; c2.state = q.state; c2.state_stride = q.state_stride; c2.ent_off = d_eoff; c2.ent_slot = d_eslot; c2.n_entries = n_entries;
+                    c2.pos = d_pos; c2.T = T; c2.o = q.o; c2.ent_chunk0 = d_echunk; c2.n_chunks = n_chunks; c2.tok = q.tok; c2.sbuf = (float*)s->lin_sbuf.p;
+                    c2.nbuf = (float*)s->lin_nbuf.p; c2.cmeta = (float*)s->lin_cm.p;
+                    kr_sv_lin_chunked(c2, st);
+                } else if (lin_chunked && kr_sv_lin_scan_wide_fits(q.kind, q.dim)) kr_sv_lin_scan_wide(q, st);
+                else kr_sv_lin_scan(q, st);
+            }
             KrSvSsdOut so{};
             so.o = (const float*)s->lin_o.p; so.x = (const float*)s->sconv.p; so.ld_x = cc; so.z = zin; so.ld_z = l.n_h; so.D = (const float*)l.ssd_d.p; so.w = (const float*)l.ssd_norm.p;
             so.heads = d.ssd_heads; so.vdim = d.ssd_vdim; so.groups = d.ssd_norm_groups; so.eps = c.norm_eps;

@@ -179,6 +179,7 @@ struct KrSvLin {
     const float* gz; int gz_ld; const float* gz_bias; float inv_tau;                     // kind 4
     const float* dtz; int dtz_ld; const float* dt_bias; const float* a_log;              // kind 5
     int norm_shared;                 // norm_w is [vdim], shared by the heads
+    int prepped;                     // kr_sv_lin_chunked: z already holds q, k as the block launches read them and tok the log decays (kr_sv_ssd_expand)
     float* z; int ld;                // [T, ld] f32: q [heads * dim] | k [heads * dim] | v [heads * vdim] | g [heads * vdim] | (mlstm) z_i [heads] | z_f [heads]
     int heads, dim, vdim, rot_dims;
     const float2* cs;                // rotation table of the step [T, rot_dims / 2] (pairs (i, i + rot_dims / 2))
@@ -209,6 +210,9 @@ bool kr_sv_lin_scan_wide_fits(int kind, int dim);
 void kr_sv_lin_scan_wide(const KrSvLin& a, hipStream_t st);
 bool kr_sv_lin_chunked_fits(int dim, int vdim);
 void kr_sv_lin_chunked(const KrSvLin& a, hipStream_t st);
+// the state-space recurrence (kind 5 fields of `a`) written as a retention with a decay per token: z_out [T, ldz] = per head [q = C | k = dt B | v = x] in
+// the recurrent mixers' layout, a.tok[t][head].x = the token's log decay.  Follow with kr_sv_lin_chunked on a kind-2 description with prepped = 1.
+void kr_sv_ssd_expand(const KrSvLin& a, float* z_out, int ldz, hipStream_t st);
 void kr_sv_lin_out(const KrSvLin& a, bool f32, hipStream_t st);
 // the selective state-space mixer after its scan: y = (o + D_h x) * silu(z), rms-normed in `groups` equal parts of the inner row, times w, times scale,
 // rounded to the storage type at out[t * out_ld + c]

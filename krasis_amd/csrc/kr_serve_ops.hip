@@ -1304,6 +1304,22 @@ __global__ void __launch_bounds__(256) sv_lin_scanw_kernel(const KrSvLin a) {
     for (int r = 0; r < DP; r++)
         if (r < dpr && part * dpr + r < dim && cv) Sg[r] = S[r];
 }
+// State-space mixer -> the block form of the recurrences: its recurrence is a retention whose decay changes from token to token,
+// S_t = e^{l_t} S_(t-1) + (dt_t B_t) x_t^T with l_t = -e^{A_h} dt_t, read out by C_t.  One wave per (token, head) writes the head's own rows
+// [q = C of its group | k = dt B of its group | v = x] where the block launches expect them and the token's log decay where sv_lin_prep_kernel would.
+__global__ void __launch_bounds__(64) sv_ssd_expand_kernel(const KrSvLin a, float* __restrict__ zo, int ldz) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, H = a.heads, N = a.dim, dv = a.vdim, hq = h / a.qk_group;
+    const float z = a.dtz[(size_t)t * a.dtz_ld + h] + a.dt_bias[h];
+    const float dt = fmaxf(z, 0.0f) + log1pf(expf(-fabsf(z)));      // softplus
+    const size_t r = (size_t)t * a.src_ld;
+    float* o = zo + (size_t)t * ldz;
+    for (int d = lane; d < N; d += 64) {
+        o[(size_t)h * N + d] = a.qsrc[r + (size_t)hq * N + d];
+        o[(size_t)H * N + (size_t)h * N + d] = a.ksrc[r + (size_t)hq * N + d] * dt;
+    }
+    for (int c = lane; c < dv; c += 64) o[(size_t)2 * H * N + (size_t)h * dv + c] = a.vsrc[r + (size_t)h * dv + c];
+    if (lane == 0) a.tok[(size_t)t * H + h] = make_float4(-expf(a.a_log[h]) * dt, 0.0f, 0.0f, 0.0f);
+}
 // gla: the decays themselves from their logits, in place: a = sigmoid(z + b)^(1 / tau), formed through the logarithm
 __global__ void sv_gla_decay_kernel(float* __restrict__ gz, const float* __restrict__ bias, size_t n, int cols, float inv_tau) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1924,11 +1940,15 @@ void kr_sv_lin_scan_wide(const KrSvLin& a, hipStream_t st) {
 #undef SV_LW
 }
 bool kr_sv_lin_chunked_fits(int dim, int vdim) { return dim <= 128 && vdim <= 128; }
+void kr_sv_ssd_expand(const KrSvLin& a, float* z_out, int ldz, hipStream_t st) {
+    if (a.T <= 0) return;
+    hipLaunchKernelGGL(sv_ssd_expand_kernel, dim3(a.T, a.heads), dim3(64), 0, st, a, z_out, ldz);
+}
 void kr_sv_lin_chunked(const KrSvLin& a, hipStream_t st) {
     if (a.T <= 0 || a.n_entries <= 0 || a.n_chunks <= 0) return;
     const bool ml = a.kind == 3;
     const int ncb = (a.vdim + 15) / 16, ndt = (a.dim + 15) / 16, ndg = (ndt + 1) / 2;
-    hipLaunchKernelGGL(sv_lin_prep_kernel, dim3(a.T, a.heads), dim3(64), 0, st, a);
+    if (!a.prepped) hipLaunchKernelGGL(sv_lin_prep_kernel, dim3(a.T, a.heads), dim3(64), 0, st, a);
     if (ml) {
         hipLaunchKernelGGL(sv_lin_mlocal_kernel<true>, dim3(a.n_chunks, a.heads), dim3(64), 0, st, a);
         hipLaunchKernelGGL(sv_lin_mchain_kernel, dim3(a.n_entries, (a.heads + 63) / 64), dim3(64), 0, st, a);
