@@ -680,17 +680,17 @@ def lufozen_serve_engine(z, kinds, ff):
     """A Lufozen model with random bf16 weights on the batched serving store at the layer sizes z (ARCH_SIZES); kinds: one letter per layer, A = attention
     (biased projections, three-tap convolution on q / k / v, per-head norms, rotation on half of a head with banded scaling, zero-score sink, element-wise
     gate), P = attention and a state-space mixer side by side (state-space heads: the size's head count, head size as channels, 128 states in 8 groups,
-    four taps), G = gla (the size's heads, keys and values of the head size, decay projections of rank 16).  Every layer: an un-gated squared-relu
+    four taps), G = gla (the size's heads, keys and values of the head size, decay projections of rank 32).  Every layer: an un-gated squared-relu
     feed-forward of ff columns.  The second and third layer form a block that runs twice."""
     from krasis_amd import model_registry as R, scheduler as SCH, serve_store as S
     W, H, G, D, V, P = (z[c] for c in ("width", "heads", "kv_heads", "dim", "vocab", "prompt"))
-    rot = dict(rot_dims=D // 2, rot_base=5e5, rot_scaling=S.ROT_BANDS, rot_factor=8.0, rot_original=8192.0, rot_fast=4.0, rot_slow=1.0)
+    rot = dict(rot_dims=D // 2, rot_base=1e6, rot_scaling=S.ROT_BANDS, rot_factor=16.0, rot_original=8192.0, rot_fast=8.0, rot_slow=2.0)
     mlp = dict(mlp_kind=S.MLP_DENSE, ff=ff, dense_act=S.ACT_RELU2)
     mk = {"A": lambda: S.LayerSpec(heads=H, kv_heads=G, dim=D, vdim=D, qk_unit_norm=S.QKNORM_WEIGHTED, scale=D ** -0.5, has_sink=S.SINK_ZERO, proj_bias=2, proj_conv=3,
                                    out_gate=S.OGATE_ELEM_SIGMOID, rot_interleaved=1, **rot, **mlp),
           "P": lambda: S.LayerSpec(heads=H, kv_heads=G, dim=D, vdim=D, qk_unit_norm=S.QKNORM_WEIGHTED, scale=D ** -0.5, rot_interleaved=0, side_mixer=S.MIX_SSD, ssd_heads=H,
-                                   ssd_vdim=D, ssd_state=128, ssd_groups=min(8, H), ssd_conv=4, ssd_norm_groups=min(8, H), mix_scale=0.6, side_scale=0.5, **rot, **mlp),
-          "G": lambda: S.LayerSpec(heads=H, kv_heads=H, dim=D, vdim=D, mixer_kind=S.MIX_GLA, lin_norm_weight=2, decay_rank=16, decay_tau=16.0, **mlp)}
+                                   ssd_vdim=D, ssd_state=128, ssd_groups=min(8, H), ssd_conv=4, ssd_norm_groups=min(8, H), mix_scale=0.75, side_scale=0.4, **rot, **mlp),
+          "G": lambda: S.LayerSpec(heads=H, kv_heads=H, dim=D, vdim=D, mixer_kind=S.MIX_GLA, lin_norm_weight=2, decay_rank=32, decay_tau=8.0, **mlp)}
     layers = [mk[c]() for c in kinds]
     if len(layers) >= 3:          # layers 1 and 2 run twice: [0, 1, 2, 1', 2', 3 ...]
         again = [mk[c]() for c in kinds[1:3]]
@@ -698,8 +698,8 @@ def lufozen_serve_engine(z, kinds, ff):
             l.weights_of = 2 + j
         layers[1].pre_add = 1; again[0].pre_add = 1
         layers = layers[:3] + again + layers[3:]
-    spec = R.ServeModelSpec(V, W, S.NORM_RMS, 1e-5, layers, None, block_kind=S.BLOCK_SEQUENTIAL, pre_norm=1, post_norm=0, norm_bias=0, embed_scale=16.0, norm_weight_offset=1.0,
-                            embed_norm=1, bigram=(4093, 31, 17), logit_scale=0.5)
+    spec = R.ServeModelSpec(V, W, S.NORM_RMS, 1e-5, layers, None, block_kind=S.BLOCK_SEQUENTIAL, pre_norm=1, post_norm=0, norm_bias=0, embed_scale=8.0, norm_weight_offset=1.0,
+                            embed_norm=1, bigram=(4093, 37, 19), logit_scale=0.25)
     eng = SCH.BatchEngine(spec, dtype="bfloat16", max_tokens=4 * (P + 256), max_slots=4)
     eng.load_synthetic(seed=7, amp=1.0)
     return eng, len(layers)
@@ -722,7 +722,7 @@ def arch_compare_lufozen(args):
         w_ff = 2 * W * ff                                             # up and down
         w_att = (2 * H * D + 2 * G * D) * W + W * H * D               # q, k, v, the element-wise gate, the output projection
         w_par = (H * D + 2 * G * D) * W + (2 * H * D + 2 * SG * N + H) * W + W * 2 * H * D
-        w_gla = 4 * H * D * W + 16 * W + H * D * 16 + W * H * D
+        w_gla = 4 * H * D * W + 32 * W + H * D * 32 + W * H * D
         att_flops = 2.0 * 2 * H * D * sum(i + 1 for i in range(P))   # causal, no window
         rec_flops = {"P": 4.0 * P * H * D * N, "G": 5.0 * P * H * D * D}
         state = {"P": H * D * N, "G": H * D * D}

@@ -50,13 +50,13 @@ def cfg_varied():
 
 
 def cfg_wide():
-    """rows that are multiples of 16 bytes and head shapes of the matrix-instruction attention (four and two heads per key head, heads of 64 and 128); the
+    """rows that are multiples of 16 bytes and head shapes of the matrix-instruction attention (four heads per key head and one, heads of 64 and 128); the
     repeated block opens the model and runs three times; recurrent heads of 64 keys; state-space heads of 32 channels over 16 states"""
-    return O.make_config(width=128, vocab=260, eps=1e-6, embed_scale=8.0, bigram=(97, 31, 17), logit_scale=0.5, loop=(0, 2, 3), layers=[
+    return O.make_config(width=128, vocab=260, eps=1e-6, embed_scale=8.0, bigram=(97, 29, 23), logit_scale=0.8, loop=(0, 2, 3), layers=[
         O.layer(O.attn(8, 2, 64, 64, scale=0.15, conv=4, rot=O.rot(32, 1e4, factor=8.0, low=1.0, high=4.0, original=128)), O.dense(96)),
-        O.layer(O.parallel(O.left(8, 4, 128, 32, scale=0.09, rot=O.rot(64, 1e5, factor=4.0, low=1.0, high=4.0, original=256)), O.ssd(4, 32, 16, groups=2, conv=4, norm_groups=2),
-                           0.6, 0.5), O.dense(64)),
-        O.layer(O.gla(2, 64, 64, tau=16.0), None),
+        O.layer(O.parallel(O.left(8, 2, 128, 64, scale=0.09, rot=O.rot(32, 1e5, factor=4.0, low=1.0, high=4.0, original=256)), O.ssd(4, 32, 16, groups=2, conv=4, norm_groups=2),
+                           0.7, 0.4), O.dense(64)),
+        O.layer(O.gla(2, 64, 64, tau=12.0), None),
         O.layer(O.attn(16, 16, 32, 32, scale=0.2, conv=2), O.dense(160)),
     ])
 
