@@ -1255,42 +1255,57 @@ __global__ void __launch_bounds__(256) sv_lin_scanw_kernel(const KrSvLin a) {
         if (more) fetch(tb + TB);
         const float* buf = lds + b * per;
         const float* qs = buf; const float* ks = qs + TB * dimp; const float* as = ks + TB * dimp; const float* vs = buf + (GLA ? 3 : 2) * TB * dimp; const float* gs = vs + TB * NC;
-        // one token: the lane's rows of q, k and the decays come from LDS (16-byte reads when the lane's rows fill DP), the state stays in registers
-        auto token = [&](int tt) -> float {
+        // The walk, written as a pipeline: the lane's rows of q, k and the decays of token tt + 1 are read from LDS (16-byte reads when the lane's rows
+        // fill DP) before token tt is worked on, and a token leaves only its lane's partial sum -- the exchanges among the 32 parts of a column are done
+        // for all 16 tokens together afterwards, as 16 independent chains.  The state stays in registers; only S is carried from token to token.
+        float qn[DP], kn[DP], dn[DP], vn = 0.0f, g0n = 1.0f, g1n = 1.0f;
+        auto read = [&](int tt) {
             const float* qp = qs + tt * dimp + part * pitch; const float* kp = ks + tt * dimp + part * pitch; const float* ap = as + tt * dimp + part * pitch;
-            float qv[DP], kv[DP], dv[DP];
             if (dpr == DP) {
 #pragma unroll
                 for (int r = 0; r < DP; r += 4) {
                     const float4 q4 = *reinterpret_cast<const float4*>(qp + r), k4 = *reinterpret_cast<const float4*>(kp + r);
-                    qv[r] = q4.x; qv[r + 1] = q4.y; qv[r + 2] = q4.z; qv[r + 3] = q4.w; kv[r] = k4.x; kv[r + 1] = k4.y; kv[r + 2] = k4.z; kv[r + 3] = k4.w;
-                    if constexpr (GLA) { const float4 a4 = *reinterpret_cast<const float4*>(ap + r); dv[r] = a4.x; dv[r + 1] = a4.y; dv[r + 2] = a4.z; dv[r + 3] = a4.w; }
+                    qn[r] = q4.x; qn[r + 1] = q4.y; qn[r + 2] = q4.z; qn[r + 3] = q4.w; kn[r] = k4.x; kn[r + 1] = k4.y; kn[r + 2] = k4.z; kn[r + 3] = k4.w;
+                    if constexpr (GLA) { const float4 a4 = *reinterpret_cast<const float4*>(ap + r); dn[r] = a4.x; dn[r + 1] = a4.y; dn[r + 2] = a4.z; dn[r + 3] = a4.w; }
                 }
             } else {
 #pragma unroll
-                for (int r = 0; r < DP; r++) { qv[r] = r < dpr ? qp[r] : 0.0f; kv[r] = r < dpr ? kp[r] : 0.0f; if constexpr (GLA) dv[r] = r < dpr ? ap[r] : 0.0f; }
+                for (int r = 0; r < DP; r++) { qn[r] = r < dpr ? qp[r] : 0.0f; kn[r] = r < dpr ? kp[r] : 0.0f; if constexpr (GLA) dn[r] = r < dpr ? ap[r] : 0.0f; }
             }
-            float av = 1.0f, bvv = vs[tt * NC + cl];
-            if constexpr (SSD) { bvv *= gs[2 * tt]; av = gs[2 * tt + 1]; }
-            float po0 = 0.0f, po1 = 0.0f;
-#pragma unroll
-            for (int r = 0; r < DP; r += 2) {
-                if constexpr (GLA) { S[r] = __builtin_fmaf(kv[r], bvv, dv[r] * S[r]); S[r + 1] = __builtin_fmaf(kv[r + 1], bvv, dv[r + 1] * S[r + 1]); }
-                else { S[r] = __builtin_fmaf(kv[r], bvv, av * S[r]); S[r + 1] = __builtin_fmaf(kv[r + 1], bvv, av * S[r + 1]); }
-                po0 = __builtin_fmaf(S[r], qv[r], po0); po1 = __builtin_fmaf(S[r + 1], qv[r + 1], po1);
-            }
-            float po = po0 + po1;
-            po += SV_DPPF(po, KR_DPP_XOR1); po += SV_DPPF(po, KR_DPP_XOR2); po += SV_DPPF(po, KR_DPP_HALF_MIRROR); po += SV_DPPF(po, KR_DPP_MIRROR);
-            return po + __shfl_xor(po, 16);
+            vn = vs[tt * NC + cl];
+            if constexpr (SSD) { g0n = gs[2 * tt]; g1n = gs[2 * tt + 1]; }
         };
         float outv[TB];
-        if (nt == TB) {
+        read(0);
+        auto walk = [&](auto full) {             // full: all 16 tokens of the batch exist -- no branch anywhere in the walk
 #pragma unroll
-            for (int tt = 0; tt < TB; tt++) outv[tt] = token(tt);
-        } else {
+        for (int tt = 0; tt < TB; tt++) {
+            float qv[DP], kv[DP], dv[DP];
 #pragma unroll
-            for (int tt = 0; tt < TB; tt++) outv[tt] = tt < nt ? token(tt) : 0.0f;
+            for (int r = 0; r < DP; r++) { qv[r] = qn[r]; kv[r] = kn[r]; dv[r] = dn[r]; }
+            const float av = g1n, bvv = SSD ? vn * g0n : vn;
+            if (tt + 1 < TB) read(tt + 1);       // rows past the portion's end are zeros in LDS: walking them leaves S unchanged only if they are skipped below
+            float po0 = 0.0f, po1 = 0.0f;
+            if (decltype(full)::value || tt < nt) {
+#pragma unroll
+                for (int r = 0; r < DP; r += 2) {
+                    if constexpr (GLA) { S[r] = __builtin_fmaf(kv[r], bvv, dv[r] * S[r]); S[r + 1] = __builtin_fmaf(kv[r + 1], bvv, dv[r + 1] * S[r + 1]); }
+                    else { S[r] = __builtin_fmaf(kv[r], bvv, av * S[r]); S[r + 1] = __builtin_fmaf(kv[r + 1], bvv, av * S[r + 1]); }
+                    po0 = __builtin_fmaf(S[r], qv[r], po0); po1 = __builtin_fmaf(S[r + 1], qv[r + 1], po1);
+                }
+            }
+            outv[tt] = po0 + po1;
         }
+        };
+        if (nt == TB) walk(std::true_type{}); else walk(std::false_type{});
+#pragma unroll
+        for (int tt = 0; tt < TB; tt++) {
+            float po = outv[tt];
+            po += SV_DPPF(po, KR_DPP_XOR1); po += SV_DPPF(po, KR_DPP_XOR2); po += SV_DPPF(po, KR_DPP_HALF_MIRROR); po += SV_DPPF(po, KR_DPP_MIRROR);
+            outv[tt] = po;
+        }
+#pragma unroll
+        for (int tt = 0; tt < TB; tt++) outv[tt] += __shfl_xor(outv[tt], 16);
         if (more) stash(lds + (b ^ 1) * per, tb + TB);
         // the outputs leave after the registers of the next batch have gone to LDS: the wait for those loads then has no younger store before it
         if (part == 0 && cv) {
