@@ -1213,13 +1213,21 @@ __global__ void __launch_bounds__(256) sv_lin_scanw_kernel(const KrSvLin a) {
     // batch; scales, masks and the gates' functions are applied when the registers go to LDS
     float pq[2 * DP], pk[2 * DP], pa[2 * DP], pv = 0.0f, pg = 0.0f;
     const int ft = tid >> 4, fd = tid & 15;
+    int gd[2 * DP], li[2 * DP];              // per staged element: its column in the head's row (clamped) and its place in an LDS buffer
+    unsigned real = 0;                       // bit j: the element exists (rows past dim are staged as zeros)
+#pragma unroll
+    for (int j = 0; j < 2 * DP; j++) {
+        const int d = fd + 16 * j, pp = dpr == DP ? d / DP : d / dpr;
+        gd[j] = min(d, dim - 1); li[j] = ft * dimp + pp * pitch + (d - pp * dpr);
+        if (d < dim) real |= 1u << j;
+    }
     auto fetch = [&](int tb) {               // global -> registers
         const int nt = min(TB, t1 - tb), tok = tb + min(ft, nt - 1);
         const size_t rb = (size_t)tok * a.src_ld + (size_t)hq * dim;
 #pragma unroll
         for (int j = 0; j < 2 * DP; j++) {
             if (j < 2 * dpr) {
-                const int d = min(fd + 16 * j, dim - 1);
+                const int d = gd[j];
                 pq[j] = a.qsrc[rb + d]; pk[j] = a.ksrc[rb + d];
                 if constexpr (GLA) pa[j] = a.gz[(size_t)tok * a.gz_ld + (size_t)h * dim + d];
             }
@@ -1234,8 +1242,8 @@ __global__ void __launch_bounds__(256) sv_lin_scanw_kernel(const KrSvLin a) {
 #pragma unroll
         for (int j = 0; j < 2 * DP; j++)
             if (j < 2 * dpr) {
-                const int d = fd + 16 * j, pp = dpr == DP ? d / DP : d / dpr, idx = ft * dimp + pp * pitch + (d - pp * dpr);
-                const bool ok = ft < nt && d < dim;
+                const int idx = li[j];
+                const bool ok = ft < nt && ((real >> j) & 1u);
                 qs[idx] = ok ? pq[j] * a.q_scale : 0.0f; ks[idx] = ok ? pk[j] * a.k_scale : 0.0f;
                 if constexpr (GLA) as[idx] = ok ? pa[j] : 0.0f;
             }
@@ -1258,43 +1266,55 @@ __global__ void __launch_bounds__(256) sv_lin_scanw_kernel(const KrSvLin a) {
         // The walk, written as a pipeline: the lane's rows of q, k and the decays of token tt + 1 are read from LDS (16-byte reads when the lane's rows
         // fill DP) before token tt is worked on, and a token leaves only its lane's partial sum -- the exchanges among the 32 parts of a column are done
         // for all 16 tokens together afterwards, as 16 independent chains.  The state stays in registers; only S is carried from token to token.
-        float qn[DP], kn[DP], dn[DP], vn = 0.0f, g0n = 1.0f, g1n = 1.0f;
-        auto read = [&](int tt) {
-            const float* qp = qs + tt * dimp + part * pitch; const float* kp = ks + tt * dimp + part * pitch; const float* ap = as + tt * dimp + part * pitch;
-            if (dpr == DP) {
+        constexpr int G = DP <= 4 ? 4 : (DP <= 8 ? 2 : 1);      // tokens read from LDS together, one group ahead of the group that is worked on
+        float qn[G][DP], kn[G][DP], dn[G][DP], vn[G], g0n[G], g1n[G];
+        auto read = [&](int t0g) {
 #pragma unroll
-                for (int r = 0; r < DP; r += 4) {
-                    const float4 q4 = *reinterpret_cast<const float4*>(qp + r), k4 = *reinterpret_cast<const float4*>(kp + r);
-                    qn[r] = q4.x; qn[r + 1] = q4.y; qn[r + 2] = q4.z; qn[r + 3] = q4.w; kn[r] = k4.x; kn[r + 1] = k4.y; kn[r + 2] = k4.z; kn[r + 3] = k4.w;
-                    if constexpr (GLA) { const float4 a4 = *reinterpret_cast<const float4*>(ap + r); dn[r] = a4.x; dn[r + 1] = a4.y; dn[r + 2] = a4.z; dn[r + 3] = a4.w; }
+            for (int j = 0; j < G; j++) {
+                const int tt = t0g + j;
+                const float* qp = qs + tt * dimp + part * pitch; const float* kp = ks + tt * dimp + part * pitch; const float* ap = as + tt * dimp + part * pitch;
+                if (dpr == DP) {
+#pragma unroll
+                    for (int r = 0; r < DP; r += 4) {
+                        const float4 q4 = *reinterpret_cast<const float4*>(qp + r), k4 = *reinterpret_cast<const float4*>(kp + r);
+                        qn[j][r] = q4.x; qn[j][r + 1] = q4.y; qn[j][r + 2] = q4.z; qn[j][r + 3] = q4.w; kn[j][r] = k4.x; kn[j][r + 1] = k4.y; kn[j][r + 2] = k4.z; kn[j][r + 3] = k4.w;
+                        if constexpr (GLA) { const float4 a4 = *reinterpret_cast<const float4*>(ap + r); dn[j][r] = a4.x; dn[j][r + 1] = a4.y; dn[j][r + 2] = a4.z; dn[j][r + 3] = a4.w; }
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < DP; r++) { qn[j][r] = r < dpr ? qp[r] : 0.0f; kn[j][r] = r < dpr ? kp[r] : 0.0f; if constexpr (GLA) dn[j][r] = r < dpr ? ap[r] : 0.0f; }
                 }
-            } else {
-#pragma unroll
-                for (int r = 0; r < DP; r++) { qn[r] = r < dpr ? qp[r] : 0.0f; kn[r] = r < dpr ? kp[r] : 0.0f; if constexpr (GLA) dn[r] = r < dpr ? ap[r] : 0.0f; }
+                vn[j] = vs[tt * NC + cl];
+                g0n[j] = SSD ? gs[2 * tt] : 1.0f; g1n[j] = SSD ? gs[2 * tt + 1] : 1.0f;
             }
-            vn = vs[tt * NC + cl];
-            if constexpr (SSD) { g0n = gs[2 * tt]; g1n = gs[2 * tt + 1]; }
         };
         float outv[TB];
         read(0);
         auto walk = [&](auto full) {             // full: all 16 tokens of the batch exist -- no branch anywhere in the walk
 #pragma unroll
-        for (int tt = 0; tt < TB; tt++) {
-            float qv[DP], kv[DP], dv[DP];
+        for (int tg = 0; tg < TB; tg += G) {
+            float qv[G][DP], kv[G][DP], dv[G][DP], av[G], bvv[G];
 #pragma unroll
-            for (int r = 0; r < DP; r++) { qv[r] = qn[r]; kv[r] = kn[r]; dv[r] = dn[r]; }
-            const float av = g1n, bvv = SSD ? vn * g0n : vn;
-            if (tt + 1 < TB) read(tt + 1);       // rows past the portion's end are zeros in LDS: walking them leaves S unchanged only if they are skipped below
-            float po0 = 0.0f, po1 = 0.0f;
-            if (decltype(full)::value || tt < nt) {
+            for (int j = 0; j < G; j++) {
 #pragma unroll
-                for (int r = 0; r < DP; r += 2) {
-                    if constexpr (GLA) { S[r] = __builtin_fmaf(kv[r], bvv, dv[r] * S[r]); S[r + 1] = __builtin_fmaf(kv[r + 1], bvv, dv[r + 1] * S[r + 1]); }
-                    else { S[r] = __builtin_fmaf(kv[r], bvv, av * S[r]); S[r + 1] = __builtin_fmaf(kv[r + 1], bvv, av * S[r + 1]); }
-                    po0 = __builtin_fmaf(S[r], qv[r], po0); po1 = __builtin_fmaf(S[r + 1], qv[r + 1], po1);
-                }
+                for (int r = 0; r < DP; r++) { qv[j][r] = qn[j][r]; kv[j][r] = kn[j][r]; dv[j][r] = dn[j][r]; }
+                av[j] = g1n[j]; bvv[j] = SSD ? vn[j] * g0n[j] : vn[j];
             }
-            outv[tt] = po0 + po1;
+            if (tg + G < TB) read(tg + G);
+#pragma unroll
+            for (int j = 0; j < G; j++) {
+                const int tt = tg + j;
+                float po0 = 0.0f, po1 = 0.0f;
+                if (decltype(full)::value || tt < nt) {
+#pragma unroll
+                    for (int r = 0; r < DP; r += 2) {
+                        if constexpr (GLA) { S[r] = __builtin_fmaf(kv[j][r], bvv[j], dv[j][r] * S[r]); S[r + 1] = __builtin_fmaf(kv[j][r + 1], bvv[j], dv[j][r + 1] * S[r + 1]); }
+                        else { S[r] = __builtin_fmaf(kv[j][r], bvv[j], av[j] * S[r]); S[r + 1] = __builtin_fmaf(kv[j][r + 1], bvv[j], av[j] * S[r + 1]); }
+                        po0 = __builtin_fmaf(S[r], qv[j][r], po0); po1 = __builtin_fmaf(S[r + 1], qv[j][r + 1], po1);
+                    }
+                }
+                outv[tt] = po0 + po1;
+            }
         }
         };
         if (nt == TB) walk(std::true_type{}); else walk(std::false_type{});
