@@ -1189,7 +1189,10 @@ __global__ void __launch_bounds__(64) sv_lin_scan_kernel(const KrSvLin a) {
 // of two LDS buffers: the loads of the next 16 are issued before the current 16 are walked and land in registers meanwhile (one barrier per 16
 // tokens); the walk itself has no branch and no store (the 16 outputs of a lane leave together afterwards), so the LDS reads of the following tokens
 // are in flight while one is worked on.  a.gz holds the decays themselves (sv_gla_decay_kernel).
-template <int KIND, int DP>
+// PIPE: the walk as an explicit pipeline (the next token's rows are read before the current one is worked on, the lane exchanges of all 16 tokens are done
+// together afterwards) -- shorter when a workgroup has its compute unit to itself; with several workgroups per compute unit the plain walk (token after
+// token, each with its own exchanges) leaves more of the issue slots to the others and the launch is over sooner.
+template <int KIND, int DP, bool PIPE>
 __global__ void __launch_bounds__(256) sv_lin_scanw_kernel(const KrSvLin a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int TB = 16, NC = 8;           // tokens per batch, value columns per workgroup
@@ -1263,12 +1266,15 @@ __global__ void __launch_bounds__(256) sv_lin_scanw_kernel(const KrSvLin a) {
         if (more) fetch(tb + TB);
         const float* buf = lds + b * per;
         const float* qs = buf; const float* ks = qs + TB * dimp; const float* as = ks + TB * dimp; const float* vs = buf + (GLA ? 3 : 2) * TB * dimp; const float* gs = vs + TB * NC;
+        float outv[TB];
+        if constexpr (PIPE) {
         // The walk, written as a pipeline: the lane's rows of q, k and the decays of token tt + 1 are read from LDS (16-byte reads when the lane's rows
         // fill DP) before token tt is worked on, and a token leaves only its lane's partial sum -- the exchanges among the 32 parts of a column are done
         // for all 16 tokens together afterwards, as 16 independent chains.  The state stays in registers; only S is carried from token to token.
-        constexpr int G = DP <= 4 ? 4 : (DP <= 8 ? 2 : 1);      // tokens read from LDS together, one group ahead of the group that is worked on
-        float qn[G][DP], kn[G][DP], dn[G][DP], vn[G], g0n[G], g1n[G];
-        auto read = [&](int t0g) {
+        constexpr int G = 1;      // tokens read from LDS together, one group ahead of the group that is worked on
+        float qq[2][G][DP], kk[2][G][DP], dd[2][G][DP], vv[2][G], g0[2][G], g1[2][G];      // two register sets, taken in turn (the loops are unrolled: every index is a constant)
+        auto read = [&](int set, int t0g) {
+            auto& qn = qq[set]; auto& kn = kk[set]; auto& dn = dd[set]; auto& vn = vv[set]; auto& g0n = g0[set]; auto& g1n = g1[set];
 #pragma unroll
             for (int j = 0; j < G; j++) {
                 const int tt = t0g + j;
@@ -1288,19 +1294,16 @@ __global__ void __launch_bounds__(256) sv_lin_scanw_kernel(const KrSvLin a) {
                 g0n[j] = SSD ? gs[2 * tt] : 1.0f; g1n[j] = SSD ? gs[2 * tt + 1] : 1.0f;
             }
         };
-        float outv[TB];
-        read(0);
+        read(0, 0);
         auto walk = [&](auto full) {             // full: all 16 tokens of the batch exist -- no branch anywhere in the walk
 #pragma unroll
         for (int tg = 0; tg < TB; tg += G) {
-            float qv[G][DP], kv[G][DP], dv[G][DP], av[G], bvv[G];
+            const int cur = (tg / G) & 1;
+            if (tg + G < TB) read(cur ^ 1, tg + G);
+            auto& qv = qq[cur]; auto& kv = kk[cur]; auto& dv = dd[cur];
+            float av[G], bvv[G];
 #pragma unroll
-            for (int j = 0; j < G; j++) {
-#pragma unroll
-                for (int r = 0; r < DP; r++) { qv[j][r] = qn[j][r]; kv[j][r] = kn[j][r]; dv[j][r] = dn[j][r]; }
-                av[j] = g1n[j]; bvv[j] = SSD ? vn[j] * g0n[j] : vn[j];
-            }
-            if (tg + G < TB) read(tg + G);
+            for (int j = 0; j < G; j++) { av[j] = g1[cur][j]; bvv[j] = SSD ? vv[cur][j] * g0[cur][j] : vv[cur][j]; }
 #pragma unroll
             for (int j = 0; j < G; j++) {
                 const int tt = tg + j;
@@ -1326,6 +1329,43 @@ __global__ void __launch_bounds__(256) sv_lin_scanw_kernel(const KrSvLin a) {
         }
 #pragma unroll
         for (int tt = 0; tt < TB; tt++) outv[tt] += __shfl_xor(outv[tt], 16);
+        } else {
+        // one token: the lane's rows of q, k and the decays come from LDS (16-byte reads when the lane's rows fill DP), the state stays in registers
+        auto token = [&](int tt) -> float {
+            const float* qp = qs + tt * dimp + part * pitch; const float* kp = ks + tt * dimp + part * pitch; const float* ap = as + tt * dimp + part * pitch;
+            float qv[DP], kv[DP], dv[DP];
+            if (dpr == DP) {
+#pragma unroll
+                for (int r = 0; r < DP; r += 4) {
+                    const float4 q4 = *reinterpret_cast<const float4*>(qp + r), k4 = *reinterpret_cast<const float4*>(kp + r);
+                    qv[r] = q4.x; qv[r + 1] = q4.y; qv[r + 2] = q4.z; qv[r + 3] = q4.w; kv[r] = k4.x; kv[r + 1] = k4.y; kv[r + 2] = k4.z; kv[r + 3] = k4.w;
+                    if constexpr (GLA) { const float4 a4 = *reinterpret_cast<const float4*>(ap + r); dv[r] = a4.x; dv[r + 1] = a4.y; dv[r + 2] = a4.z; dv[r + 3] = a4.w; }
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < DP; r++) { qv[r] = r < dpr ? qp[r] : 0.0f; kv[r] = r < dpr ? kp[r] : 0.0f; if constexpr (GLA) dv[r] = r < dpr ? ap[r] : 0.0f; }
+            }
+            float av = 1.0f, bvv = vs[tt * NC + cl];
+            if constexpr (SSD) { bvv *= gs[2 * tt]; av = gs[2 * tt + 1]; }
+            float po0 = 0.0f, po1 = 0.0f;
+#pragma unroll
+            for (int r = 0; r < DP; r += 2) {
+                if constexpr (GLA) { S[r] = __builtin_fmaf(kv[r], bvv, dv[r] * S[r]); S[r + 1] = __builtin_fmaf(kv[r + 1], bvv, dv[r + 1] * S[r + 1]); }
+                else { S[r] = __builtin_fmaf(kv[r], bvv, av * S[r]); S[r + 1] = __builtin_fmaf(kv[r + 1], bvv, av * S[r + 1]); }
+                po0 = __builtin_fmaf(S[r], qv[r], po0); po1 = __builtin_fmaf(S[r + 1], qv[r + 1], po1);
+            }
+            float po = po0 + po1;
+            po += SV_DPPF(po, KR_DPP_XOR1); po += SV_DPPF(po, KR_DPP_XOR2); po += SV_DPPF(po, KR_DPP_HALF_MIRROR); po += SV_DPPF(po, KR_DPP_MIRROR);
+            return po + __shfl_xor(po, 16);
+        };
+        if (nt == TB) {
+#pragma unroll
+            for (int tt = 0; tt < TB; tt++) outv[tt] = token(tt);
+        } else {
+#pragma unroll
+            for (int tt = 0; tt < TB; tt++) outv[tt] = tt < nt ? token(tt) : 0.0f;
+        }
+        }
         if (more) stash(lds + (b ^ 1) * per, tb + TB);
         // the outputs leave after the registers of the next batch have gone to LDS: the wait for those loads then has no younger store before it
         if (part == 0 && cv) {
@@ -1967,11 +2007,15 @@ void kr_sv_lin_scan_wide(const KrSvLin& a, hipStream_t st) {
         const size_t n = (size_t)a.T * a.heads * a.dim;
         hipLaunchKernelGGL(sv_gla_decay_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, const_cast<float*>(a.gz), a.gz_bias, n, a.heads * a.dim, a.inv_tau);
     }
-#define SV_LW(K_, DP_) do { if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)sv_lin_scanw_kernel<K_, DP_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
-                            hipLaunchKernelGGL((sv_lin_scanw_kernel<K_, DP_>), grid, dim3(256), lds, st, a); } while (0)
-#define SV_LW_D(K_) do { if (dpr <= 4) SV_LW(K_, 4); else if (dpr <= 8) SV_LW(K_, 8); else SV_LW(K_, 16); } while (0)
+    // one workgroup per compute unit or fewer: the pipelined walk; more: the plain one (256 compute units, up to three workgroups on each)
+    const bool pipe = (size_t)grid.x * grid.y * grid.z <= 384;
+#define SV_LW(K_, DP_, P_) do { if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)sv_lin_scanw_kernel<K_, DP_, P_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+                                hipLaunchKernelGGL((sv_lin_scanw_kernel<K_, DP_, P_>), grid, dim3(256), lds, st, a); } while (0)
+#define SV_LW_P(K_, DP_) do { if (pipe) SV_LW(K_, DP_, true); else SV_LW(K_, DP_, false); } while (0)
+#define SV_LW_D(K_) do { if (dpr <= 4) SV_LW_P(K_, 4); else if (dpr <= 8) SV_LW_P(K_, 8); else SV_LW_P(K_, 16); } while (0)
     if (a.kind == 4) SV_LW_D(4); else SV_LW_D(5);
 #undef SV_LW_D
+#undef SV_LW_P
 #undef SV_LW
 }
 bool kr_sv_lin_chunked_fits(int dim, int vdim) { return dim <= 128 && vdim <= 128; }

@@ -565,3 +565,19 @@ def test_state_space_mixer_as_a_layers_only_mixer():
     assert rel(whole, ref) < 2e-4
     rows = [eng.step([("d", toks[:7], [6])])[0][0]] + [eng.step([("d", [t], [0])])[0][0] for t in toks[7:]]
     assert rel(np.stack(rows), ref[6:]) < 2e-4
+
+
+def test_many_workgroups_take_the_plain_walk_of_the_scan():
+    """four prompts in one step, seven heads of 112 value columns: more workgroups than the pipelined form of the prompt scan is launched for, in the gla
+    mixer and in a state-space mixer whose 130 states are beyond the block form"""
+    cfg = small_model([O.layer(O.gla(7, 8, 112, tau=5.0), None),
+                       O.layer(O.parallel(O.left(2, 1, 8, 8), O.ssd(7, 112, 130, groups=7, conv=2, norm_groups=1), 0.5, 0.8), O.dense(24))])
+    W = O.random_weights(cfg, 51)
+    seqs = {k: tokens(cfg, n, 52 + i) for i, (k, n) in enumerate((("a", 40), ("b", 33), ("c", 57), ("d", 36)))}
+    eng = engine(cfg, W, max_tokens=512)
+    lg, _ = eng.step([(k, t, [len(t) - 1, 0]) for k, t in seqs.items()])
+    ref = np.concatenate([O.forward(cfg, W, t)[0][[len(t) - 1, 0]] for t in seqs.values()])
+    assert rel(lg, ref) < 2e-4
+    nxt, _ = eng.step([(k, [5], [0]) for k in seqs])        # the states the plain walk left continue in the decode form
+    ref = np.stack([O.forward(cfg, W, t + [5])[0][-1] for t in seqs.values()])
+    assert rel(nxt, ref) < 2e-4
